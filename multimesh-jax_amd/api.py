@@ -1,0 +1,385 @@
+"""Host-side mirror of the reference's reshard interface over the C ABI.
+
+Names and argument meaning follow the reference's C++ surface for this path:
+the descriptor functions of src/pjrt_client/mm_sharding.{h,cc} and the store
+subset of xla::ZukuExecuteContext (src/pjrt_client/zuku_execute_context.h:38-133).
+Everything here is a thin ctypes call into libmmreshard.so; no arithmetic of the
+path is done in Python and there is no fallback when the library or the GPU is
+missing.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Dict, Iterable, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+from . import _binding as B
+from ._binding import MmrError  # noqa: F401  (re-export)
+
+ITEMSIZE = {name: None for name in B.DTYPES}
+
+
+def itemsize(element_type: str) -> int:
+    return B.load().mmr_itemsize(B.DTYPES[element_type])
+
+
+# --------------------------------------------------------------------------
+# descriptors
+# --------------------------------------------------------------------------
+def sharded_shape(type: str, dims: Sequence[Tuple[int, int, int]], dev_start: int, dev_count: int,
+                  minor_to_major: Optional[Sequence[int]] = None) -> B.ShardedShape:
+    """zuku::ShardedShape{type, sharding{dims{size, sharding, permutation}, devices{start, num_devices}}}."""
+    if len(dims) > B.MMR_MAX_DIMS:
+        raise ValueError("at most %d descriptor entries" % B.MMR_MAX_DIMS)
+    s = B.ShardedShape()
+    s.dtype = B.DTYPES[type]
+    s.ndims = len(dims)
+    for i, (size, sharding, permutation) in enumerate(dims):
+        s.dims[i] = B.ShardingDim(size, sharding, permutation)
+    s.dev_start, s.dev_count = dev_start, dev_count
+    if minor_to_major is not None:
+        s.has_layout = 1
+        for i, m in enumerate(minor_to_major):
+            s.minor_to_major[i] = m
+    return s
+
+
+def describe(s: B.ShardedShape) -> dict:
+    d = {"type": B.DTYPE_NAMES.get(s.dtype, s.dtype),
+         "dims": [[s.dims[i].size, s.dims[i].sharding, s.dims[i].permutation] for i in range(s.ndims)],
+         "dev_start": s.dev_start, "dev_count": s.dev_count}
+    if s.has_layout:
+        d["minor_to_major"] = [s.minor_to_major[i] for i in range(s.ndims)]
+    return d
+
+
+def op_sharding(type: str = "OTHER", tile_dims: Sequence[int] = (), iota_reshape_dims: Sequence[int] = (),
+                iota_transpose_perm: Sequence[int] = (), tile_assignment_devices: Sequence[int] = (),
+                replicate_on_last_tile_dim: bool = False, iota_offset: int = 0) -> B.OpSharding:
+    o = B.OpSharding()
+    o.type = B.SHARDING_TYPES[type]
+    o.n_tile_dims = len(tile_dims)
+    for i, t in enumerate(tile_dims):
+        o.tile_dims[i] = t
+    o.n_iota_dims = len(iota_reshape_dims)
+    for i, t in enumerate(iota_reshape_dims):
+        o.iota_reshape_dims[i] = t
+    perm = list(iota_transpose_perm) or list(range(len(iota_reshape_dims)))
+    for i, t in enumerate(perm):
+        o.iota_transpose_perm[i] = t
+    o.replicate_on_last_tile_dim = int(replicate_on_last_tile_dim)
+    o.iota_offset = iota_offset
+    if tile_assignment_devices:
+        arr = (C.c_int64 * len(tile_assignment_devices))(*tile_assignment_devices)
+        o._keepalive = arr
+        o.tile_assignment_devices = C.cast(arr, C.POINTER(C.c_int64))
+        o.n_devices = len(tile_assignment_devices)
+    return o
+
+
+def _i64(values: Sequence[int]):
+    return (C.c_int64 * max(len(values), 1))(*values)
+
+
+def ComputeIndexSet(global_index: int, dims: Sequence[int]) -> List[int]:
+    out = _i64([0] * len(dims))
+    B.check(B.load().mmr_compute_index_set(global_index, _i64(dims), len(dims), out))
+    return list(out)[:len(dims)]
+
+
+def ComputeGlobalIndex(indices: Sequence[int], dims: Sequence[int]) -> int:
+    out = C.c_int64()
+    B.check(B.load().mmr_compute_global_index(_i64(indices), _i64(dims), len(dims), C.byref(out)))
+    return out.value
+
+
+def LogicalToPhysicalSharding(logical_to_device_axes: Sequence[Sequence[int]], devices: Tuple[int, int],
+                              dims: Sequence[int], list_all_devices: bool = False) -> B.OpSharding:
+    flat: List[int] = []
+    begin = [0]
+    for axes in logical_to_device_axes:
+        flat.extend(axes)
+        begin.append(len(flat))
+    out = B.OpSharding()
+    B.check(B.load().mmr_logical_to_physical_sharding(
+        (C.c_int32 * max(len(flat), 1))(*flat), (C.c_int32 * len(begin))(*begin), len(logical_to_device_axes),
+        devices[0], devices[1], _i64(dims), len(dims), int(list_all_devices), C.byref(out)))
+    return out
+
+
+def TileAssignmentDevices(op: B.OpSharding) -> List[int]:
+    n = 1
+    for i in range(op.n_tile_dims):
+        n *= op.tile_dims[i]
+    out = _i64([0] * n)
+    got = C.c_int64()
+    B.check(B.load().mmr_tile_assignment_devices(C.byref(op), out, n, C.byref(got)))
+    return list(out)[:got.value]
+
+
+def CanonicalizeSharding(op: B.OpSharding, shape: Sequence[int], element_type: str,
+                         shape_is_global: bool = True) -> B.ShardedShape:
+    out = B.ShardedShape()
+    B.check(B.load().mmr_canonicalize_sharding(C.byref(op), _i64(shape), len(shape), B.DTYPES[element_type],
+                                               int(shape_is_global), C.byref(out)))
+    return out
+
+
+def XlaShapeToZukuShape(shape: Sequence[int], element_type: str, devices: Tuple[int, int], op: B.OpSharding,
+                        shape_is_global: bool = True) -> B.ShardedShape:
+    out = B.ShardedShape()
+    B.check(B.load().mmr_xla_shape_to_sharded_shape(_i64(shape), len(shape), B.DTYPES[element_type], devices[0],
+                                                    devices[1], C.byref(op), int(shape_is_global), C.byref(out)))
+    return out
+
+
+def MeshEquivalentSharding(lhs: B.OpSharding, rhs: B.OpSharding) -> bool:
+    out = C.c_int32()
+    B.check(B.load().mmr_mesh_equivalent_sharding(C.byref(lhs), C.byref(rhs), C.byref(out)))
+    return bool(out.value)
+
+
+def NeedsReshard(operand_devices: Tuple[int, int], devices: Tuple[int, int], operand_sharding: B.OpSharding,
+                 sharding: B.OpSharding) -> bool:
+    out = C.c_int32()
+    B.check(B.load().mmr_needs_reshard(operand_devices[0], operand_devices[1], devices[0], devices[1],
+                                       C.byref(operand_sharding), C.byref(sharding), C.byref(out)))
+    return bool(out.value)
+
+
+def shard_extents(s: B.ShardedShape) -> Tuple[int, ...]:
+    ext = _i64([0] * B.MMR_MAX_DIMS)
+    rank = C.c_int32()
+    B.check(B.load().mmr_shard_extents(C.byref(s), ext, C.byref(rank)))
+    return tuple(ext[i] for i in range(rank.value))
+
+
+def shard_bytes(s: B.ShardedShape) -> int:
+    out = C.c_int64()
+    B.check(B.load().mmr_shard_bytes(C.byref(s), C.byref(out)))
+    return out.value
+
+
+def device_of_tile(s: B.ShardedShape, coord: Sequence[int]) -> int:
+    out = C.c_int64()
+    B.check(B.load().mmr_device_of_tile(C.byref(s), _i64(coord), C.byref(out)))
+    return out.value
+
+
+def tile_of_device(s: B.ShardedShape, device: int) -> List[int]:
+    out = _i64([0] * B.MMR_MAX_DIMS)
+    B.check(B.load().mmr_tile_of_device(C.byref(s), device, out))
+    return [out[i] for i in range(s.ndims)]
+
+
+# --------------------------------------------------------------------------
+# plans (host only)
+# --------------------------------------------------------------------------
+def _shape_array(shapes: Sequence[B.ShardedShape]):
+    arr = (B.ShardedShape * max(len(shapes), 1))()
+    for i, s in enumerate(shapes):
+        arr[i] = s
+    return arr
+
+
+class Plan:
+    """Copy plan of one or more (source, destination) descriptor pairs."""
+
+    def __init__(self, srcs: Sequence[B.ShardedShape], dsts: Sequence[B.ShardedShape],
+                 chunk_bytes: int = 0, order: int = 0):
+        if isinstance(srcs, B.ShardedShape):
+            srcs, dsts = [srcs], [dsts]
+        self._lib = B.load()
+        self._h = C.c_void_p()
+        opt = B.PlanOptions(chunk_bytes, order)
+        B.check(self._lib.mmr_plan_create(_shape_array(srcs), _shape_array(dsts), len(srcs), C.byref(opt),
+                                          C.byref(self._h)))
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.mmr_plan_destroy(self._h)
+            self._h = None
+
+    @property
+    def stats(self) -> dict:
+        st = B.PlanStats()
+        B.check(self._lib.mmr_plan_get_stats(self._h, C.byref(st)))
+        return st.as_dict()
+
+    def copy_chunks(self, kind: int) -> np.ndarray:
+        """kind 0: 16-byte aligned chunks, kind 1: generic chunks (structured array)."""
+        n = self._lib.mmr_plan_get_copy_chunks(self._h, kind, None, 0)
+        buf = (B.CopyChunk * max(n, 1))()
+        self._lib.mmr_plan_get_copy_chunks(self._h, kind, buf, n)
+        return np.frombuffer(buf, dtype=np.dtype(B.CopyChunk), count=n).copy()
+
+    def transpose_chunks(self) -> np.ndarray:
+        n = self._lib.mmr_plan_get_transpose_chunks(self._h, None, 0)
+        buf = (B.TransposeChunk * max(n, 1))()
+        self._lib.mmr_plan_get_transpose_chunks(self._h, buf, n)
+        return np.frombuffer(buf, dtype=np.dtype(B.TransposeChunk), count=n).copy()
+
+    def slot_bases(self) -> List[int]:
+        n = self._lib.mmr_plan_get_slot_bases(self._h, None, 0)
+        buf = _i64([0] * n)
+        self._lib.mmr_plan_get_slot_bases(self._h, buf, n)
+        return list(buf)[:n]
+
+
+# --------------------------------------------------------------------------
+# execution
+# --------------------------------------------------------------------------
+class StoreHandle:
+    """One sharded array: a buffer per device of its device list (store_handle_fwd.h:15-19)."""
+
+    def __init__(self, ctx: "ReshardContext", handle: C.c_void_p, shape: B.ShardedShape, name: str):
+        self._ctx = ctx
+        self._h = handle
+        self.shape = shape
+        self.name = name
+        self.unique_id = B.load().mmr_store_id(handle)
+
+    @property
+    def devices(self) -> range:
+        return range(self.shape.dev_start, self.shape.dev_start + self.shape.dev_count)
+
+    @property
+    def shard_bytes(self) -> int:
+        return shard_bytes(self.shape)
+
+
+class ReshardContext:
+    """Store subset of xla::ZukuExecuteContext on one MI355X.
+
+    Every logical device is a separate buffer in this GPU's HBM, so the
+    per-device arguments of the reference (local_device_id, global_device_id)
+    become an explicit `device` where one shard is meant and disappear where the
+    reference call is control-replicated over the devices.
+    """
+
+    def __init__(self, hip_device: int = 0, hip_stream: Optional[int] = None):
+        self._lib = B.load()
+        self._h = C.c_void_p()
+        B.check(self._lib.mmr_context_create(hip_device, C.c_void_p(hip_stream) if hip_stream else None,
+                                             C.byref(self._h)))
+
+    def close(self) -> None:
+        if self._h:
+            self._lib.mmr_context_destroy(self._h)
+            self._h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    # -- stores -----------------------------------------------------------
+    def CreateStore(self, shape: B.ShardedShape, name: Optional[str] = None,
+                    allocate_from_cache: bool = False) -> StoreHandle:
+        h = C.c_void_p()
+        flags = B.MMR_STORE_FROM_CACHE if allocate_from_cache else 0
+        B.check(self._lib.mmr_store_create(self._h, C.byref(shape), name.encode() if name else None, flags,
+                                           C.byref(h)))
+        return StoreHandle(self, h, shape, name or "anonymous")
+
+    def AssembleShards(self, shape: B.ShardedShape, device: int, data, existing_store: Optional[StoreHandle] = None,
+                       size: Optional[int] = None) -> StoreHandle:
+        """Shard{data, local_device_id, size}: `data` is a NumPy array (host) or an int device pointer."""
+        store = existing_store if existing_store is not None else self.CreateStore(shape)
+        if isinstance(data, np.ndarray):
+            arr = np.ascontiguousarray(data)
+            B.check(self._lib.mmr_store_assemble(self._h, store._h, device, arr.ctypes.data, arr.nbytes, 0))
+        else:
+            if size is None:
+                raise ValueError("size is required for a device pointer")
+            B.check(self._lib.mmr_store_assemble(self._h, store._h, device, C.c_void_p(int(data)), size, 1))
+        return store
+
+    def SliceLocalShard(self, device: int, store: StoreHandle, wait: bool = True) -> int:
+        p = C.c_void_p()
+        fn = self._lib.mmr_store_shard_ptr if wait else self._lib.mmr_store_shard_ptr_async
+        B.check(fn(self._h, store._h, device, C.byref(p)))
+        return p.value or 0
+
+    def ReadShard(self, store: StoreHandle, device: int, dtype=np.uint8) -> np.ndarray:
+        """Host copy of one shard's bytes (what ToLiteral reads through SliceLocalShard)."""
+        out = np.empty(store.shard_bytes, dtype=np.uint8)
+        B.check(self._lib.mmr_store_read_shard(self._h, store._h, device, out.ctypes.data, out.nbytes))
+        return out.view(dtype)
+
+    def HasLocalShard(self, store: StoreHandle, device: int) -> bool:
+        out = C.c_int32()
+        B.check(self._lib.mmr_store_has_shard(store._h, device, C.byref(out)))
+        return bool(out.value)
+
+    def GetStoreShardedShape(self, store: StoreHandle) -> B.ShardedShape:
+        out = B.ShardedShape()
+        B.check(self._lib.mmr_store_get_shape(store._h, C.byref(out)))
+        return out
+
+    def Free(self, store: StoreHandle, keep_in_cache: bool = False) -> None:
+        B.check(self._lib.mmr_store_free(self._h, store._h, int(keep_in_cache)))
+        store._h = None
+
+    def Destroy(self, store: StoreHandle) -> None:
+        self.Free(store, keep_in_cache=False)
+
+    def ClearStoreCache(self) -> None:
+        B.check(self._lib.mmr_clear_store_cache(self._h))
+
+    # -- the hot path -----------------------------------------------------
+    def Reshard(self, src: StoreHandle, dst: StoreHandle) -> None:
+        B.check(self._lib.mmr_reshard(self._h, src._h, dst._h))
+
+    def ReshardBatch(self, srcs: Sequence[StoreHandle], dsts: Sequence[StoreHandle]) -> None:
+        n = len(srcs)
+        if n != len(dsts):
+            raise ValueError("as many destinations as sources")
+        key = (tuple(s.unique_id for s in srcs), tuple(d.unique_id for d in dsts))
+        cached = getattr(self, "_batch_args", None)
+        if cached is None or cached[0] != key:
+            sa = (C.c_void_p * max(n, 1))(*[s._h for s in srcs])
+            da = (C.c_void_p * max(n, 1))(*[d._h for d in dsts])
+            self._batch_args = cached = (key, sa, da)
+        B.check(self._lib.mmr_reshard_batch(self._h, cached[1], cached[2], n))
+
+    def Sync(self) -> None:
+        B.check(self._lib.mmr_sync(self._h))
+
+    # -- measurement and inspection ----------------------------------------
+    def set_plan_options(self, chunk_bytes: int = 0, order: int = 0) -> None:
+        opt = B.PlanOptions(chunk_bytes, order)
+        B.check(self._lib.mmr_context_set_plan_options(self._h, C.byref(opt)))
+
+    def StartTimer(self) -> None:
+        B.check(self._lib.mmr_timer_start(self._h))
+
+    def StopTimer(self) -> float:
+        ms = C.c_float()
+        B.check(self._lib.mmr_timer_stop(self._h, C.byref(ms)))
+        return ms.value
+
+    @property
+    def stream(self) -> int:
+        p = C.c_void_p()
+        B.check(self._lib.mmr_context_stream(self._h, C.byref(p)))
+        return p.value or 0
+
+    @property
+    def stats(self) -> dict:
+        st = B.ContextStats()
+        B.check(self._lib.mmr_context_get_stats(self._h, C.byref(st)))
+        return st.as_dict()
+
+    def plan_stats(self, src: StoreHandle, dst: StoreHandle) -> dict:
+        st = B.PlanStats()
+        B.check(self._lib.mmr_reshard_plan_stats(self._h, src._h, dst._h, C.byref(st)))
+        return st.as_dict()

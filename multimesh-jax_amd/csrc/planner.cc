@@ -1,0 +1,394 @@
+// Shard-intersection planner (host only).
+//
+// For every destination tile the overlapping source tiles are found by
+// per-dimension interval intersection; each overlap is an N-d box with a byte
+// stride per dim on either side.  Boxes are canonicalised (extent-1 dims
+// dropped, dims that are contiguous on both sides merged) and lowered to
+// workgroup-sized chunks:
+//   * copy chunks     - n2 x n1 rows of w contiguous bytes (minor dim kept),
+//   * transpose chunks - <=64x64-element tiles staged through LDS (source and
+//                        destination disagree on the minor dim),
+//   * fill chunks      - copy chunks without a source, zeroing the pad of short
+//                        edge tiles.
+#include "planner.h"
+
+#include <algorithm>
+#include <cstring>
+
+namespace mmr {
+namespace {
+
+struct BoxDim {
+  int64_t n;  // extent in elements
+  int64_t s;  // source byte stride
+  int64_t d;  // destination byte stride
+};
+
+int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+class Builder {
+ public:
+  Builder(mmr_plan* plan, uint32_t chunk_bytes) : plan_(plan), chunk_bytes_(chunk_bytes) {}
+
+  void add_box(uint32_t src_slot, uint32_t dst_slot, int64_t src_off, int64_t dst_off, const BoxDim* in, int rank,
+               int itemsize) {
+    std::vector<BoxDim> dims;
+    int64_t volume = 1;
+    for (int i = 0; i < rank; ++i) {
+      if (in[i].n <= 0) return;
+      volume *= in[i].n;
+      if (in[i].n > 1) dims.push_back(in[i]);
+    }
+    const bool fill = src_slot == MMR_SLOT_FILL;
+    if (fill) {
+      plan_->stats.bytes_filled += volume * itemsize;
+    } else {
+      plan_->stats.bytes_moved += volume * itemsize;
+      plan_->stats.n_boxes += 1;
+    }
+    // destination-major order, then merge dims that are contiguous on both sides
+    std::stable_sort(dims.begin(), dims.end(), [](const BoxDim& a, const BoxDim& b) {
+      return a.d != b.d ? a.d > b.d : a.s > b.s;
+    });
+    for (int i = static_cast<int>(dims.size()) - 1; i > 0; --i) {
+      if (dims[i - 1].s == dims[i].s * dims[i].n && dims[i - 1].d == dims[i].d * dims[i].n) {
+        dims[i - 1] = BoxDim{dims[i - 1].n * dims[i].n, dims[i].s, dims[i].d};
+        dims.erase(dims.begin() + i);
+      }
+    }
+    int run = -1, x = -1, y = -1;
+    for (int i = 0; i < static_cast<int>(dims.size()); ++i) {
+      if (dims[i].s == itemsize && dims[i].d == itemsize) run = i;
+      else if (dims[i].s == itemsize) x = i;
+      else if (dims[i].d == itemsize) y = i;
+    }
+    if (run < 0 && x >= 0 && y >= 0 && !fill) {
+      lower_transpose(src_slot, dst_slot, src_off, dst_off, dims, x, y, itemsize);
+      return;
+    }
+    int64_t w = itemsize;
+    if (run >= 0) {
+      w = dims[run].n * itemsize;
+      dims.erase(dims.begin() + run);
+    }
+    lower_copy(src_slot, dst_slot, src_off, dst_off, dims, w, fill);
+  }
+
+ private:
+  // index of the dim whose rows are closest together on either side
+  static int pick_row_dim(const std::vector<BoxDim>& dims, int skip) {
+    int best = -1;
+    for (int i = 0; i < static_cast<int>(dims.size()); ++i) {
+      if (i == skip) continue;
+      if (best < 0) { best = i; continue; }
+      const int64_t a_lo = std::min(dims[i].s, dims[i].d), a_hi = std::max(dims[i].s, dims[i].d);
+      const int64_t b_lo = std::min(dims[best].s, dims[best].d), b_hi = std::max(dims[best].s, dims[best].d);
+      if (a_lo < b_lo || (a_lo == b_lo && a_hi < b_hi)) best = i;
+    }
+    return best;
+  }
+
+  // Calls fn(src_delta, dst_delta) for every index combination of `dims`.
+  template <class Fn>
+  static void for_each_index(const std::vector<BoxDim>& dims, Fn&& fn) {
+    std::vector<int64_t> idx(dims.size(), 0);
+    int64_t so = 0, dof = 0;
+    while (true) {
+      fn(so, dof);
+      int k = static_cast<int>(dims.size()) - 1;
+      for (; k >= 0; --k) {
+        idx[k]++;
+        so += dims[k].s;
+        dof += dims[k].d;
+        if (idx[k] < dims[k].n) break;
+        so -= dims[k].s * dims[k].n;
+        dof -= dims[k].d * dims[k].n;
+        idx[k] = 0;
+      }
+      if (k < 0) break;
+    }
+  }
+
+  void emit_copy(uint32_t src_slot, uint32_t dst_slot, int64_t so, int64_t dof, int64_t w, int64_t n1, int64_t n2,
+                 int64_t s1, int64_t d1, int64_t s2, int64_t d2, bool fill) {
+    mmr_copy_chunk c{};
+    c.src_slot = src_slot;
+    c.dst_slot = dst_slot;
+    c.src_off = fill ? 0 : static_cast<uint64_t>(so);
+    c.dst_off = static_cast<uint64_t>(dof);
+    c.w = static_cast<uint32_t>(w);
+    c.n1 = static_cast<uint32_t>(n1);
+    c.n2 = static_cast<uint32_t>(n2);
+    c.s1 = (n1 > 1 && !fill) ? s1 : 0;
+    c.d1 = n1 > 1 ? d1 : 0;
+    c.s2 = (n2 > 1 && !fill) ? s2 : 0;
+    c.d2 = n2 > 1 ? d2 : 0;
+    uint64_t bits = c.src_off | c.dst_off | c.w | static_cast<uint64_t>(c.s1) | static_cast<uint64_t>(c.d1) |
+                    static_cast<uint64_t>(c.s2) | static_cast<uint64_t>(c.d2);
+    c.align = (bits & 15u) ? static_cast<uint32_t>(bits & (~bits + 1)) : 16u;
+    if (fill) plan_->stats.n_fill_chunks += 1;
+    (c.align == 16 ? plan_->copy16 : plan_->generic).push_back(c);
+  }
+
+  void lower_copy(uint32_t src_slot, uint32_t dst_slot, int64_t so, int64_t dof, std::vector<BoxDim>& outer, int64_t w,
+                  bool fill) {
+    const int64_t cb = chunk_bytes_;
+    if (w > cb) {
+      // long rows: split columns into near-equal segments on 256-byte boundaries of the row
+      const int64_t nseg = ceil_div(w, cb);
+      const int64_t seg = ceil_div(ceil_div(w, nseg), 256) * 256;
+      for_each_index(outer, [&](int64_t ds, int64_t dd) {
+        for (int64_t c0 = 0; c0 < w; c0 += seg)
+          emit_copy(src_slot, dst_slot, so + ds + c0, dof + dd + c0, std::min(seg, w - c0), 1, 1, 0, 0, 0, 0, fill);
+      });
+      return;
+    }
+    const int64_t rows = std::max<int64_t>(1, cb / w);
+    int i1 = pick_row_dim(outer, -1);
+    if (i1 < 0) {
+      emit_copy(src_slot, dst_slot, so, dof, w, 1, 1, 0, 0, 0, 0, fill);
+      return;
+    }
+    const BoxDim dim1 = outer[i1];
+    const int64_t n1 = std::min(dim1.n, rows);
+    BoxDim dim2{1, 0, 0};
+    int64_t n2 = 1;
+    int i2 = -1;
+    if (n1 == dim1.n && rows / n1 >= 2) {
+      i2 = pick_row_dim(outer, i1);
+      if (i2 >= 0) {
+        dim2 = outer[i2];
+        n2 = std::min(dim2.n, rows / n1);
+      }
+    }
+    std::vector<BoxDim> rest;
+    for (int i = 0; i < static_cast<int>(outer.size()); ++i)
+      if (i != i1 && i != i2) rest.push_back(outer[i]);
+    for_each_index(rest, [&](int64_t ds, int64_t dd) {
+      for (int64_t b2 = 0; b2 < dim2.n; b2 += n2) {
+        const int64_t m2 = std::min(n2, dim2.n - b2);
+        for (int64_t b1 = 0; b1 < dim1.n; b1 += n1) {
+          const int64_t m1 = std::min(n1, dim1.n - b1);
+          emit_copy(src_slot, dst_slot, so + ds + b2 * dim2.s + b1 * dim1.s, dof + dd + b2 * dim2.d + b1 * dim1.d, w, m1,
+                    m2, dim1.s, dim1.d, dim2.s, dim2.d, fill);
+        }
+      }
+    });
+  }
+
+  void lower_transpose(uint32_t src_slot, uint32_t dst_slot, int64_t so, int64_t dof, const std::vector<BoxDim>& dims,
+                       int x, int y, int itemsize) {
+    const int64_t tile = itemsize == 16 ? kTransposeTile / 2 : kTransposeTile;
+    const BoxDim dx = dims[x], dy = dims[y];
+    std::vector<BoxDim> outer;
+    for (int i = 0; i < static_cast<int>(dims.size()); ++i)
+      if (i != x && i != y) outer.push_back(dims[i]);
+    int ib = pick_row_dim(outer, -1);
+    BoxDim db{1, 0, 0};
+    if (ib >= 0) {
+      db = outer[ib];
+      outer.erase(outer.begin() + ib);
+    }
+    const int64_t nb = std::max<int64_t>(1, std::min<int64_t>(db.n, chunk_bytes_ / (tile * tile * itemsize)));
+    for_each_index(outer, [&](int64_t ds, int64_t dd) {
+      for (int64_t b0 = 0; b0 < db.n; b0 += nb) {
+        for (int64_t y0 = 0; y0 < dy.n; y0 += tile) {
+          for (int64_t x0 = 0; x0 < dx.n; x0 += tile) {
+            mmr_transpose_chunk c{};
+            c.src_slot = src_slot;
+            c.dst_slot = dst_slot;
+            c.src_off = static_cast<uint64_t>(so + ds + b0 * db.s + y0 * dy.s + x0 * dx.s);
+            c.dst_off = static_cast<uint64_t>(dof + dd + b0 * db.d + y0 * dy.d + x0 * dx.d);
+            c.nx = static_cast<uint32_t>(std::min(tile, dx.n - x0));
+            c.ny = static_cast<uint32_t>(std::min(tile, dy.n - y0));
+            c.nb = static_cast<uint32_t>(std::min(nb, db.n - b0));
+            c.itemsize = static_cast<uint32_t>(itemsize);
+            c.src_ystride = dy.s;
+            c.dst_xstride = dx.d;
+            c.src_bstride = db.s;
+            c.dst_bstride = db.d;
+            plan_->transposes.push_back(c);
+          }
+        }
+      }
+    });
+  }
+
+  mmr_plan* plan_;
+  uint32_t chunk_bytes_;
+};
+
+int plan_one_array(Builder& b, const Side& S, const Side& D, uint32_t slot_base) {
+  const int rank = S.rank;
+  const int item = S.itemsize;
+  for (int i = 0; i < rank; ++i)
+    if (S.size[i] == 0) return MMR_OK;  // empty array: nothing to move, nothing to pad
+  for (int64_t dd = 0; dd < D.dev_count; ++dd) {
+    const uint32_t dslot = slot_base + static_cast<uint32_t>(S.dev_count + dd);
+    int64_t lo[kMaxRank], hi[kMaxRank], valid[kMaxRank];
+    bool padded = false, empty = false;
+    for (int i = 0; i < rank; ++i) {
+      const int64_t c = (dd / D.dev_stride[i]) % D.tiles[i];
+      lo[i] = std::min(c * D.ext[i], D.size[i]);
+      hi[i] = std::min(lo[i] + D.ext[i], D.size[i]);
+      valid[i] = hi[i] - lo[i];
+      padded |= valid[i] < D.ext[i];
+      empty |= valid[i] == 0;
+    }
+    if (padded) {
+      // the pad of a short tile is rank slabs: dim i beyond its valid extent,
+      // dims before it inside theirs, dims after it whole
+      for (int i = 0; i < rank; ++i) {
+        if (valid[i] == D.ext[i]) continue;
+        BoxDim dims[kMaxRank];
+        for (int j = 0; j < rank; ++j) {
+          const int64_t n = j < i ? valid[j] : (j == i ? D.ext[i] - valid[i] : D.ext[j]);
+          dims[j] = BoxDim{n, D.stride[j] * item, D.stride[j] * item};
+        }
+        b.add_box(MMR_SLOT_FILL, dslot, 0, valid[i] * D.stride[i] * item, dims, rank, item);
+      }
+    }
+    if (empty) continue;
+    int64_t t_lo[kMaxRank], t_n[kMaxRank], combos = 1;
+    for (int i = 0; i < rank; ++i) {
+      t_lo[i] = lo[i] / S.ext[i];
+      t_n[i] = (hi[i] - 1) / S.ext[i] - t_lo[i] + 1;
+      combos *= t_n[i];
+    }
+    for (int64_t c = 0; c < combos; ++c) {
+      int64_t rem = c, sdev = 0, soff = 0, doff = 0;
+      BoxDim dims[kMaxRank];
+      for (int i = rank - 1; i >= 0; --i) {
+        const int64_t t = t_lo[i] + rem % t_n[i];
+        rem /= t_n[i];
+        const int64_t s_lo = t * S.ext[i];
+        const int64_t b_lo = std::max(lo[i], s_lo);
+        const int64_t b_hi = std::min(hi[i], std::min(s_lo + S.ext[i], S.size[i]));
+        dims[i] = BoxDim{b_hi - b_lo, S.stride[i] * item, D.stride[i] * item};
+        soff += (b_lo - s_lo) * S.stride[i] * item;
+        doff += (b_lo - lo[i]) * D.stride[i] * item;
+        sdev += t * S.dev_stride[i];  // of R source replicas the lowest device id is read
+      }
+      b.add_box(slot_base + static_cast<uint32_t>(sdev), dslot, soff, doff, dims, rank, item);
+    }
+  }
+  return MMR_OK;
+}
+
+}  // namespace
+
+std::string plan_key(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int n,
+                     const mmr_plan_options& options) {
+  std::string k;
+  k.append(reinterpret_cast<const char*>(&options), sizeof(options));
+  k.append(reinterpret_cast<const char*>(&n), sizeof(n));
+  for (int a = 0; a < n; ++a) {
+    k += descriptor_key(srcs[a]);
+    k += descriptor_key(dsts[a]);
+  }
+  return k;
+}
+
+int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int n, const mmr_plan_options& options,
+               mmr_plan* plan) {
+  if (n < 0 || (n > 0 && (!srcs || !dsts))) return fail(MMR_INVALID_ARGUMENT, "bad descriptor arrays");
+  uint32_t chunk_bytes = options.chunk_bytes ? options.chunk_bytes : kDefaultChunkBytes;
+  chunk_bytes = std::min<uint32_t>(std::max<uint32_t>(chunk_bytes, 1024), 16u << 20) & ~255u;
+  plan->options = options;
+  Builder builder(plan, chunk_bytes);
+  for (int a = 0; a < n; ++a) {
+    Side S, D;
+    if (int rc = make_side(srcs[a], &S)) return rc;
+    if (int rc = make_side(dsts[a], &D)) return rc;
+    if (S.dtype != D.dtype)
+      return fail(MMR_INVALID_ARGUMENT, "array %d: source type %d differs from destination type %d", a, S.dtype, D.dtype);
+    if (S.rank != D.rank)
+      return fail(MMR_INVALID_ARGUMENT, "array %d: source rank %d differs from destination rank %d", a, S.rank, D.rank);
+    for (int i = 0; i < S.rank; ++i)
+      if (S.size[i] != D.size[i])
+        return fail(MMR_INVALID_ARGUMENT, "array %d: dim %d is %lld in the source and %lld in the destination", a, i,
+                    (long long)S.size[i], (long long)D.size[i]);
+    if (plan->n_slots + S.dev_count + D.dev_count >= static_cast<int64_t>(MMR_SLOT_FILL))
+      return fail(MMR_INVALID_ARGUMENT, "too many shard buffers in one plan");
+    plan->srcs.push_back(srcs[a]);
+    plan->dsts.push_back(dsts[a]);
+    plan->slot_bases.push_back(plan->n_slots);
+    if (int rc = plan_one_array(builder, S, D, static_cast<uint32_t>(plan->n_slots))) return rc;
+    plan->n_slots += S.dev_count + D.dev_count;
+  }
+  const uint32_t order = options.order ? options.order : 2;
+  if (order == 2 || order == 3) {
+    auto key = [order](const mmr_copy_chunk& c) {
+      return order == 2 ? std::make_pair(c.dst_slot, c.dst_off) : std::make_pair(c.src_slot, c.src_off);
+    };
+    auto cmp = [&](const mmr_copy_chunk& a, const mmr_copy_chunk& b) { return key(a) < key(b); };
+    std::stable_sort(plan->copy16.begin(), plan->copy16.end(), cmp);
+    std::stable_sort(plan->generic.begin(), plan->generic.end(), cmp);
+    std::stable_sort(plan->transposes.begin(), plan->transposes.end(),
+                     [order](const mmr_transpose_chunk& a, const mmr_transpose_chunk& b) {
+                       return order == 2 ? std::make_pair(a.dst_slot, a.dst_off) < std::make_pair(b.dst_slot, b.dst_off)
+                                         : std::make_pair(a.src_slot, a.src_off) < std::make_pair(b.src_slot, b.src_off);
+                     });
+  }
+  plan->stats.n_arrays = n;
+  plan->stats.n_copy16_chunks = static_cast<int64_t>(plan->copy16.size());
+  plan->stats.n_copy_generic_chunks = static_cast<int64_t>(plan->generic.size());
+  plan->stats.n_transpose_chunks = static_cast<int64_t>(plan->transposes.size());
+  plan->stats.n_slots = plan->n_slots;
+  plan->stats.table_bytes =
+      static_cast<int64_t>((plan->copy16.size() + plan->generic.size()) * sizeof(mmr_copy_chunk) +
+                           plan->transposes.size() * sizeof(mmr_transpose_chunk) + plan->n_slots * sizeof(void*));
+  return MMR_OK;
+}
+
+}  // namespace mmr
+
+using mmr::fail;
+
+extern "C" {
+
+int mmr_plan_create(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int32_t n_arrays,
+                    const mmr_plan_options* options, mmr_plan** out) {
+  if (!out) return fail(MMR_INVALID_ARGUMENT, "null output");
+  mmr_plan_options opt{};
+  if (options) opt = *options;
+  mmr_plan* plan = new mmr_plan();
+  if (int rc = mmr::build_plan(srcs, dsts, n_arrays, opt, plan)) {
+    delete plan;
+    return rc;
+  }
+  *out = plan;
+  return MMR_OK;
+}
+
+void mmr_plan_destroy(mmr_plan* plan) { delete plan; }
+
+int mmr_plan_get_stats(const mmr_plan* plan, mmr_plan_stats* out) {
+  if (!plan || !out) return fail(MMR_INVALID_ARGUMENT, "null argument");
+  *out = plan->stats;
+  return MMR_OK;
+}
+
+int64_t mmr_plan_get_copy_chunks(const mmr_plan* plan, int32_t kind, mmr_copy_chunk* out, int64_t capacity) {
+  if (!plan) return 0;
+  const auto& v = kind == 0 ? plan->copy16 : plan->generic;
+  int64_t n = std::min<int64_t>(capacity, static_cast<int64_t>(v.size()));
+  if (out && n > 0) std::memcpy(out, v.data(), sizeof(mmr_copy_chunk) * n);
+  return out ? n : static_cast<int64_t>(v.size());
+}
+
+int64_t mmr_plan_get_transpose_chunks(const mmr_plan* plan, mmr_transpose_chunk* out, int64_t capacity) {
+  if (!plan) return 0;
+  int64_t n = std::min<int64_t>(capacity, static_cast<int64_t>(plan->transposes.size()));
+  if (out && n > 0) std::memcpy(out, plan->transposes.data(), sizeof(mmr_transpose_chunk) * n);
+  return out ? n : static_cast<int64_t>(plan->transposes.size());
+}
+
+int64_t mmr_plan_get_slot_bases(const mmr_plan* plan, int64_t* out, int64_t capacity) {
+  if (!plan) return 0;
+  int64_t n = std::min<int64_t>(capacity, static_cast<int64_t>(plan->slot_bases.size()));
+  if (out && n > 0) std::memcpy(out, plan->slot_bases.data(), sizeof(int64_t) * n);
+  return out ? n : static_cast<int64_t>(plan->slot_bases.size());
+}
+
+}  // extern "C"

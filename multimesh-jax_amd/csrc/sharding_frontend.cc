@@ -1,0 +1,369 @@
+// Descriptor front-end (host only): how an XLA sharding plus a shape becomes the
+// sharded-shape descriptor the reshard consumes.  Follows the reference's
+// src/pjrt_client/mm_sharding.{h,cc} and mpmd_insert_reshard.cc:33-43 with the
+// XLA proto types flattened to the PODs of mmreshard.h.
+#include <algorithm>
+#include <numeric>
+#include <vector>
+
+#include "common.h"
+
+using mmr::fail;
+
+namespace {
+
+bool is_replicated(const mmr_op_sharding& s) { return s.type == MMR_SHARDING_REPLICATED; }
+bool is_maximal(const mmr_op_sharding& s) { return s.type == MMR_SHARDING_MAXIMAL; }
+
+// mm_sharding.cc:19-33
+bool replicated_on_assigned_submesh(const mmr_op_sharding& s) {
+  if (is_replicated(s)) return true;
+  if (s.replicate_on_last_tile_dim) {
+    for (int d = 0; d + 1 < s.n_tile_dims; ++d)
+      if (s.tile_dims[d] != 1) return false;
+    return true;
+  }
+  return false;
+}
+
+// mm_sharding.cc:35-38
+bool replicated_or_submesh_replicate(const mmr_op_sharding& s) {
+  return is_replicated(s) || replicated_on_assigned_submesh(s) || is_maximal(s);
+}
+
+int check_sharding(const mmr_op_sharding* s) {
+  if (!s) return fail(MMR_INVALID_ARGUMENT, "null sharding");
+  if (s->n_tile_dims < 0 || s->n_tile_dims > MMR_MAX_DIMS || s->n_iota_dims < 0 || s->n_iota_dims > MMR_MAX_DIMS)
+    return fail(MMR_INVALID_ARGUMENT, "sharding has too many dims");
+  return MMR_OK;
+}
+
+// XLA's IotaTileAssignment::Create canonical form, which is what the reference
+// walks (HloSharding::FromProto builds every assignment through it): size-1
+// iota dims are dropped and iota dims that stay adjacent and in order after the
+// transpose are merged.
+void canonical_iota(const mmr_op_sharding& s, std::vector<int64_t>* dims, std::vector<int>* perm) {
+  std::vector<int64_t> d(s.iota_reshape_dims, s.iota_reshape_dims + s.n_iota_dims);
+  std::vector<int> p(s.iota_transpose_perm, s.iota_transpose_perm + s.n_iota_dims);
+  std::vector<int> renum(d.size(), -1);
+  std::vector<int64_t> kept;
+  for (size_t i = 0; i < d.size(); ++i)
+    if (d[i] != 1) {
+      renum[i] = static_cast<int>(kept.size());
+      kept.push_back(d[i]);
+    }
+  std::vector<int> kp;
+  for (int v : p)
+    if (v >= 0 && v < static_cast<int>(renum.size()) && renum[v] >= 0) kp.push_back(renum[v]);
+  if (kept.empty()) {
+    *dims = {1};
+    *perm = {0};
+    return;
+  }
+  std::vector<std::vector<int>> groups;  // runs of consecutive iota dims, in transposed order
+  for (int v : kp) {
+    if (!groups.empty() && groups.back().back() + 1 == v) groups.back().push_back(v);
+    else groups.push_back({v});
+  }
+  std::vector<int> order(groups.size());
+  std::iota(order.begin(), order.end(), 0);
+  std::sort(order.begin(), order.end(), [&](int a, int b) { return groups[a][0] < groups[b][0]; });
+  std::vector<int> new_index(groups.size());
+  dims->clear();
+  for (size_t i = 0; i < order.size(); ++i) {
+    new_index[order[i]] = static_cast<int>(i);
+    int64_t n = 1;
+    for (int v : groups[order[i]]) n *= kept[v];
+    dims->push_back(n);
+  }
+  perm->clear();
+  for (size_t g = 0; g < groups.size(); ++g) perm->push_back(new_index[g]);
+}
+
+int map_type(int32_t dtype) {
+  // mm_sharding.cc:376-425: only these fifteen types have a runtime type
+  if (dtype < MMR_PRED || dtype > MMR_C128) return fail(MMR_UNSUPPORTED, "Unsupported type: %d", dtype);
+  return MMR_OK;
+}
+
+// mm_sharding.cc:275-432
+int canonicalize_iota(const mmr_op_sharding& s, const std::vector<int64_t>& reshape_dims, const std::vector<int>& perm,
+                      int64_t offset, const int64_t* shape, int rank, int32_t dtype, bool shape_is_global,
+                      mmr_sharded_shape* out) {
+  const int nta = s.n_tile_dims;
+  std::vector<int64_t> permuted(reshape_dims.size());
+  for (size_t i = 0; i < perm.size(); ++i) permuted[i] = reshape_dims[perm[i]];
+
+  // :297-325  tile dims that one iota dim spans form a group
+  std::vector<std::vector<int>> groups(1);
+  size_t iota_dim = 0;
+  int64_t spanned = 1;
+  int ta = 0;
+  for (; ta < nta && iota_dim < permuted.size(); ++ta) {
+    spanned *= s.tile_dims[ta];
+    const int64_t span = permuted[iota_dim];
+    if (span < s.tile_dims[ta])
+      return fail(MMR_INVALID_ARGUMENT,
+                  "CanonicalizeSharding: sharding has multiple iota dims within a single tensor dimension, which is "
+                  "not yet supported");
+    groups.back().push_back(ta);
+    if (spanned >= span) {
+      ++iota_dim;
+      if (iota_dim < permuted.size()) groups.emplace_back();
+      spanned = 1;
+    }
+  }
+  for (; ta < nta; ++ta) groups.back().push_back(ta);
+
+  // :327-339  the reference picks group transpose_perm[k] as the k-th most significant
+  std::vector<int> full;
+  for (size_t k = 0; k < perm.size(); ++k) {
+    if (perm[k] < 0 || perm[k] >= static_cast<int>(groups.size()))
+      return fail(MMR_INVALID_ARGUMENT, "CanonicalizeSharding: iota transpose does not match the tile dims");
+    for (int d : groups[perm[k]]) full.push_back(d);
+  }
+  if (static_cast<int>(full.size()) != nta)
+    return fail(MMR_INVALID_ARGUMENT, "CanonicalizeSharding: iota dims do not cover the tile dims");
+
+  // :341-369
+  const int num_shape_dims = s.replicate_on_last_tile_dim ? nta - 1 : nta;
+  if (num_shape_dims > rank) return fail(MMR_INVALID_ARGUMENT, "sharding has more tile dims than the shape has dims");
+  mmr_sharded_shape r{};
+  r.dtype = dtype;
+  r.ndims = nta;
+  for (int k = 0; k < nta; ++k) {
+    const int tdim = full[k];
+    const int64_t extent = s.tile_dims[tdim];
+    if (tdim == num_shape_dims) {
+      r.dims[tdim] = mmr_sharding_dim{1, extent, k};
+    } else {
+      int64_t size = shape[tdim];
+      if (!shape_is_global) size *= extent;
+      r.dims[tdim] = mmr_sharding_dim{size, extent, k};
+    }
+  }
+  int64_t n = 1;
+  for (int64_t d : reshape_dims) n *= d;
+  r.dev_start = offset;
+  r.dev_count = n;
+  if (int rc = map_type(dtype)) return rc;
+  *out = r;
+  return MMR_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mmr_compute_index_set(int64_t global_index, const int64_t* dims, int32_t n, int64_t* out) {
+  if (n < 0 || (n > 0 && (!dims || !out))) return fail(MMR_INVALID_ARGUMENT, "bad arguments");
+  int64_t remainder = global_index, stride = 1;
+  for (int d = 0; d < n; ++d) stride *= dims[d];
+  for (int d = 0; d < n; ++d) {
+    if (dims[d] <= 0) return fail(MMR_INVALID_ARGUMENT, "dim %d has extent %lld", d, (long long)dims[d]);
+    stride /= dims[d];
+    out[d] = remainder / stride;
+    remainder -= out[d] * stride;
+  }
+  return MMR_OK;
+}
+
+int mmr_compute_global_index(const int64_t* indices, const int64_t* dims, int32_t n, int64_t* out) {
+  if (n < 0 || !out || (n > 0 && (!dims || !indices))) return fail(MMR_INVALID_ARGUMENT, "bad arguments");
+  int64_t stride = 1, index = 0;
+  for (int d = n - 1; d >= 0; --d) {
+    index += stride * indices[d];
+    stride *= dims[d];
+  }
+  *out = index;
+  return MMR_OK;
+}
+
+int mmr_logical_to_physical_sharding(const int32_t* axes_flat, const int32_t* axes_begin, int32_t n_logical,
+                                     int64_t dev_start, int64_t dev_count, const int64_t* mesh_dims, int32_t n_mesh,
+                                     int32_t list_all_devices, mmr_op_sharding* out) {
+  (void)dev_count;
+  if (!out || n_logical < 0 || n_mesh < 0 || n_mesh > MMR_MAX_DIMS || (n_logical > 0 && !axes_begin))
+    return fail(MMR_INVALID_ARGUMENT, "bad arguments");
+  std::vector<int> used(n_mesh, 0);
+  bool fully_replicated = true;
+  for (int l = 0; l < n_logical; ++l) {
+    for (int k = axes_begin[l]; k < axes_begin[l + 1]; ++k) {
+      const int ax = axes_flat[k];
+      if (ax < 0 || ax >= n_mesh) return fail(MMR_INVALID_ARGUMENT, "device axis %d is outside the %d-axis mesh", ax, n_mesh);
+      used[ax] = 1;
+      if (mesh_dims[ax] > 1) fully_replicated = false;
+    }
+  }
+  mmr_op_sharding r{};
+  if (n_logical == 0 || (fully_replicated && !list_all_devices)) {  // :204-209
+    r.type = MMR_SHARDING_REPLICATED;
+    *out = r;
+    return MMR_OK;
+  }
+  int64_t replication = 1, total = 1;
+  bool any_unused = false;
+  for (int d = 0; d < n_mesh; ++d) {
+    if (!used[d]) {
+      any_unused = true;
+      replication *= mesh_dims[d];
+    }
+    total *= mesh_dims[d];
+  }
+  if (n_logical + (any_unused ? 1 : 0) > MMR_MAX_DIMS) return fail(MMR_INVALID_ARGUMENT, "too many tile dims");
+  std::vector<int> dim_perm;
+  for (int l = 0; l < n_logical; ++l) {
+    std::vector<int> assigned(axes_flat + axes_begin[l], axes_flat + axes_begin[l + 1]);
+    std::sort(assigned.begin(), assigned.end());
+    int64_t t = 1;
+    for (int ax : assigned) {
+      t *= mesh_dims[ax];
+      dim_perm.push_back(ax);
+    }
+    r.tile_dims[l] = t;
+  }
+  r.n_tile_dims = n_logical;
+  for (int d = 0; d < n_mesh; ++d)
+    if (!used[d]) dim_perm.push_back(d);
+  if (any_unused) r.tile_dims[r.n_tile_dims++] = replication;
+  r.type = MMR_SHARDING_OTHER;
+  bool need_perm = false;
+  for (int i = 0; i < n_mesh; ++i) need_perm |= dim_perm[i] != i;
+  if (need_perm) {
+    r.n_iota_dims = n_mesh;
+    for (int i = 0; i < n_mesh; ++i) {
+      r.iota_reshape_dims[i] = mesh_dims[i];
+      r.iota_transpose_perm[i] = dim_perm[i];
+    }
+  } else {
+    r.n_iota_dims = 1;
+    r.iota_reshape_dims[0] = total;
+    r.iota_transpose_perm[0] = 0;
+  }
+  r.replicate_on_last_tile_dim = any_unused;
+  r.iota_offset = dev_start;  // :270
+  *out = r;
+  return MMR_OK;
+}
+
+int mmr_tile_assignment_devices(const mmr_op_sharding* s, int64_t* out, int64_t capacity, int64_t* n_out) {
+  if (int rc = check_sharding(s)) return rc;
+  if (!out || !n_out) return fail(MMR_INVALID_ARGUMENT, "null output");
+  int64_t n = 1;
+  for (int d = 0; d < s->n_tile_dims; ++d) n *= s->tile_dims[d];
+  if (n > capacity) return fail(MMR_INVALID_ARGUMENT, "%lld tiles do not fit a buffer of %lld", (long long)n, (long long)capacity);
+  if (s->n_iota_dims == 0) {
+    if (s->n_devices != n || !s->tile_assignment_devices)
+      return fail(MMR_INVALID_ARGUMENT, "explicit device list has %lld entries for %lld tiles", (long long)s->n_devices, (long long)n);
+    std::copy(s->tile_assignment_devices, s->tile_assignment_devices + n, out);
+    *n_out = n;
+    return MMR_OK;
+  }
+  const int k = s->n_iota_dims;
+  int64_t total = 1, stride[MMR_MAX_DIMS];
+  for (int d = k - 1; d >= 0; --d) {
+    stride[d] = total;
+    total *= s->iota_reshape_dims[d];
+  }
+  if (total != n) return fail(MMR_INVALID_ARGUMENT, "iota dims hold %lld devices for %lld tiles", (long long)total, (long long)n);
+  // walk the transposed iota array in row-major order
+  int64_t tdims[MMR_MAX_DIMS], idx[MMR_MAX_DIMS] = {};
+  for (int d = 0; d < k; ++d) tdims[d] = s->iota_reshape_dims[s->iota_transpose_perm[d]];
+  for (int64_t i = 0; i < n; ++i) {
+    int64_t v = 0;
+    for (int d = 0; d < k; ++d) v += idx[d] * stride[s->iota_transpose_perm[d]];
+    out[i] = v + s->iota_offset;
+    for (int d = k - 1; d >= 0; --d) {
+      if (++idx[d] < tdims[d]) break;
+      idx[d] = 0;
+    }
+  }
+  *n_out = n;
+  return MMR_OK;
+}
+
+int mmr_canonicalize_sharding(const mmr_op_sharding* s, const int64_t* shape, int32_t rank, int32_t dtype,
+                              int32_t shape_is_global, mmr_sharded_shape* out) {
+  if (int rc = check_sharding(s)) return rc;
+  if (!out || rank < 0 || (rank > 0 && !shape)) return fail(MMR_INVALID_ARGUMENT, "bad arguments");
+  if (s->n_iota_dims > 0) {  // :438-441
+    std::vector<int64_t> dims;
+    std::vector<int> perm;
+    canonical_iota(*s, &dims, &perm);
+    return canonicalize_iota(*s, dims, perm, s->iota_offset, shape, rank, dtype, shape_is_global != 0, out);
+  }
+  // :443-455  an explicit list is accepted only if it counts up by one
+  if (!s->tile_assignment_devices || s->n_devices < 1)
+    return fail(MMR_INVALID_ARGUMENT, "CanonicalizeSharding: sharding has no tile assignment");
+  int64_t prev = s->tile_assignment_devices[0] - 1;
+  for (int64_t i = 0; i < s->n_devices; ++i) {
+    if (s->tile_assignment_devices[i] != prev + 1)
+      return fail(MMR_INVALID_ARGUMENT, "CanonicalizeSharding: only supported for iota tile assignment");
+    prev = s->tile_assignment_devices[i];
+  }
+  return canonicalize_iota(*s, {s->n_devices}, {0}, s->tile_assignment_devices[0], shape, rank, dtype,
+                           shape_is_global != 0, out);
+}
+
+int mmr_xla_shape_to_sharded_shape(const int64_t* shape, int32_t rank, int32_t dtype, int64_t dev_start,
+                                   int64_t dev_count, const mmr_op_sharding* s, int32_t shape_is_global,
+                                   mmr_sharded_shape* out) {
+  if (int rc = check_sharding(s)) return rc;
+  if (!out || rank < 0 || (rank > 0 && !shape)) return fail(MMR_INVALID_ARGUMENT, "bad arguments");
+  if (int rc = map_type(dtype)) return rc;  // :586-636
+  if (is_replicated(*s) || is_maximal(*s)) {  // :638-654
+    if (rank + (dev_count > 1 ? 1 : 0) > MMR_MAX_DIMS) return fail(MMR_INVALID_ARGUMENT, "rank %d is too large", rank);
+    mmr_sharded_shape r{};
+    r.dtype = dtype;
+    for (int d = 0; d < rank; ++d) r.dims[d] = mmr_sharding_dim{shape[d], 1, d};
+    r.ndims = rank;
+    if (dev_count > 1) r.dims[r.ndims++] = mmr_sharding_dim{1, dev_count, rank};
+    r.dev_start = dev_start;
+    r.dev_count = dev_count;
+    *out = r;
+    return MMR_OK;
+  }
+  mmr_sharded_shape r{};
+  if (int rc = mmr_canonicalize_sharding(s, shape, rank, dtype, shape_is_global, &r)) return rc;
+  if (r.dev_start != dev_start || r.dev_count != dev_count) {  // :659-668
+    if (r.dev_count != dev_count)
+      return fail(MMR_INVALID_ARGUMENT, "devices=[%lld...%lld) given to XlaShapeToZukuShape differs from sharding",
+                  (long long)dev_start, (long long)(dev_start + dev_count));
+    r.dev_start = dev_start;  // same-shaped meshes can be resharded across
+  }
+  *out = r;
+  return MMR_OK;
+}
+
+int mmr_mesh_equivalent_sharding(const mmr_op_sharding* lhs, const mmr_op_sharding* rhs, int32_t* out) {
+  if (int rc = check_sharding(lhs)) return rc;
+  if (int rc = check_sharding(rhs)) return rc;
+  if (!out) return fail(MMR_INVALID_ARGUMENT, "null output");
+  if (replicated_or_submesh_replicate(*lhs)) {
+    *out = replicated_or_submesh_replicate(*rhs);
+  } else if (replicated_or_submesh_replicate(*rhs)) {
+    *out = 0;
+  } else {
+    *out = lhs->n_tile_dims == rhs->n_tile_dims &&
+           std::equal(lhs->tile_dims, lhs->tile_dims + lhs->n_tile_dims, rhs->tile_dims);
+  }
+  return MMR_OK;
+}
+
+int mmr_needs_reshard(int64_t operand_dev_start, int64_t operand_dev_count, int64_t dev_start, int64_t dev_count,
+                      const mmr_op_sharding* operand_sharding, const mmr_op_sharding* sharding, int32_t* out) {
+  if (int rc = check_sharding(operand_sharding)) return rc;
+  if (int rc = check_sharding(sharding)) return rc;
+  if (!out) return fail(MMR_INVALID_ARGUMENT, "null output");
+  const bool contains = operand_dev_start <= dev_start && dev_start + dev_count <= operand_dev_start + operand_dev_count;
+  if (is_replicated(*operand_sharding) && is_replicated(*sharding) && contains) {
+    *out = 0;
+    return MMR_OK;
+  }
+  int32_t equivalent = 0;
+  if (int rc = mmr_mesh_equivalent_sharding(operand_sharding, sharding, &equivalent)) return rc;
+  *out = operand_dev_start != dev_start || operand_dev_count != dev_count || !equivalent;
+  return MMR_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,96 @@
+"""Shared test helpers: conversions between the neutral workload dicts, the
+oracle's descriptors and the library's, and a NumPy interpreter of plan tables
+(so the planner can be checked against the oracle without a GPU)."""
+from __future__ import annotations
+
+from typing import Dict, Optional, Sequence
+
+import numpy as np
+
+import multimesh_jax_amd as mm
+from oracle import reshard_oracle as ro
+from oracle.sharding_oracle import ShardedShape, ShardingDim
+
+
+def oracle_shape(type: str, side: dict) -> ShardedShape:
+    return ShardedShape(type, tuple(ShardingDim(*d) for d in side["dims"]), side["dev_start"], side["dev_count"])
+
+
+def lib_shape(type: str, side: dict):
+    return mm.sharded_shape(type, side["dims"], side["dev_start"], side["dev_count"], side.get("minor_to_major"))
+
+
+def raw_global(a: dict, g: np.ndarray) -> np.ndarray:
+    return g.view(ro.raw_dtype(a["type"]))
+
+
+def apply_plan(plan: "mm.Plan", buffers: Sequence[np.ndarray]) -> None:
+    """Executes a plan's tables on host buffers (one flat uint8 array per slot)
+    exactly as the kernels define a chunk; pure NumPy, for CPU-side checks."""
+    for kind in (0, 1):
+        for c in plan.copy_chunks(kind):
+            dst = buffers[int(c["dst_slot"])]
+            fill = int(c["src_slot"]) == 0xFFFFFFFF
+            src = None if fill else buffers[int(c["src_slot"])]
+            w = int(c["w"])
+            if kind == 0:
+                assert int(c["align"]) == 16
+            for r2 in range(int(c["n2"])):
+                for r1 in range(int(c["n1"])):
+                    do = int(c["dst_off"]) + r2 * int(c["d2"]) + r1 * int(c["d1"])
+                    assert do + w <= dst.size
+                    if fill:
+                        dst[do:do + w] = 0
+                    else:
+                        so = int(c["src_off"]) + r2 * int(c["s2"]) + r1 * int(c["s1"])
+                        assert so + w <= src.size
+                        dst[do:do + w] = src[so:so + w]
+            a = int(c["align"])
+            for v in ("dst_off", "w", "d1", "d2") + (() if fill else ("src_off", "s1", "s2")):
+                assert int(c[v]) % a == 0, (v, c)
+    for c in plan.transpose_chunks():
+        src = buffers[int(c["src_slot"])]
+        dst = buffers[int(c["dst_slot"])]
+        it = int(c["itemsize"])
+        assert int(c["nx"]) <= 64 and int(c["ny"]) <= 64
+        for b in range(int(c["nb"])):
+            for y in range(int(c["ny"])):
+                for x in range(int(c["nx"])):
+                    so = int(c["src_off"]) + b * int(c["src_bstride"]) + y * int(c["src_ystride"]) + x * it
+                    do = int(c["dst_off"]) + b * int(c["dst_bstride"]) + x * int(c["dst_xstride"]) + y * it
+                    dst[do:do + it] = src[so:so + it]
+
+
+def run_plan_on_host(arrays: Sequence[dict], globals_: Sequence[np.ndarray], chunk_bytes: int = 0,
+                     order: int = 0, poison: int = 0xA5):
+    """Returns (plan, per-array dict device -> uint8 dst buffer) after interpreting
+    the batch plan on host copies of the shards."""
+    srcs = [lib_shape(a["type"], a["src"]) for a in arrays]
+    dsts = [lib_shape(a["type"], a["dst"]) for a in arrays]
+    plan = mm.Plan(srcs, dsts, chunk_bytes=chunk_bytes, order=order)
+    bases = plan.slot_bases()
+    buffers = [None] * plan.stats["n_slots"]
+    outs = []
+    for a, g, base in zip(arrays, globals_, bases):
+        so = oracle_shape(a["type"], a["src"])
+        do = oracle_shape(a["type"], a["dst"])
+        shards = ro.make_shards(raw_global(a, g), so, a["src"].get("minor_to_major"))
+        for k in range(so.dev_count):
+            buffers[base + k] = shards[so.dev_start + k].view(np.uint8).reshape(-1)
+        nbytes = int(np.prod(ro.shard_shape(do))) * ro.ITEMSIZE[a["type"]] if ro.shard_shape(do) else ro.ITEMSIZE[a["type"]]
+        out = {}
+        for k in range(do.dev_count):
+            buf = np.full(nbytes, poison, dtype=np.uint8)
+            buffers[base + so.dev_count + k] = buf
+            out[do.dev_start + k] = buf
+        outs.append(out)
+    apply_plan(plan, buffers)
+    return plan, outs
+
+
+def oracle_outputs(a: dict, g: np.ndarray) -> Dict[int, np.ndarray]:
+    so = oracle_shape(a["type"], a["src"])
+    do = oracle_shape(a["type"], a["dst"])
+    shards = ro.make_shards(raw_global(a, g), so, a["src"].get("minor_to_major"))
+    out = ro.reshard(shards, so, do, a["src"].get("minor_to_major"), a["dst"].get("minor_to_major"))
+    return {d: v.view(np.uint8).reshape(-1) for d, v in out.items()}

@@ -1,0 +1,305 @@
+"""Parity of the HIP path with the oracle, through the C ABI, on a real MI355X.
+
+Bar: bit-exact (pure data movement; integer, byte and float bit patterns alike).
+"""
+import random
+import sys
+
+import numpy as np
+import pytest
+
+import multimesh_jax_amd as mm
+from multimesh_jax_amd import workloads
+from oracle import reshard_cpu, reshard_oracle as ro
+
+from helpers import lib_shape, oracle_outputs, oracle_shape, raw_global
+from gpu_helpers import gpu_reshard, make_stores, read_all
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print("[gpu-test] " + msg, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = mm.ReshardContext(0)
+    yield c
+    c.close()
+
+
+def _compare(arrays, gs, outs):
+    for a, g, out in zip(arrays, gs, outs):
+        expect = oracle_outputs(a, g)
+        assert sorted(out) == sorted(expect)
+        for dev in expect:
+            assert out[dev].tobytes() == expect[dev].tobytes(), (a["name"], dev)
+
+
+@pytest.mark.parametrize("index", [1, 2, 3, 5, 6])
+def test_benchmark_config_full_size(ctx, index):
+    say("config %d full size" % index)
+    arrays = workloads.config(index)
+    gs = [workloads.generate(a) for a in arrays]
+    outs = gpu_reshard(ctx, arrays, gs)
+    _compare(arrays, gs, outs)
+
+
+@pytest.mark.parametrize("chunk_bytes,order", [(4096, 1), (16384, 3), (262144, 2)])
+def test_plan_options_do_not_change_results(ctx, chunk_bytes, order):
+    say("plan options chunk=%d order=%d" % (chunk_bytes, order))
+    ctx.set_plan_options(chunk_bytes, order)
+    try:
+        for index, scale in ((2, 8), (3, 4), (5, 8)):
+            arrays = workloads.config(index, scale)
+            gs = [workloads.generate(a) for a in arrays]
+            _compare(arrays, gs, gpu_reshard(ctx, arrays, gs))
+    finally:
+        ctx.set_plan_options(0, 0)
+
+
+def test_config4_scaled_batched_bit_exact(ctx):
+    say("config 4 scale 8, one batched plan")
+    arrays = workloads.config(4, 8)
+    gs = [workloads.generate(a) for a in arrays]
+    before = ctx.stats
+    outs = gpu_reshard(ctx, arrays, gs, batch=True)
+    after = ctx.stats
+    _compare(arrays, gs, outs)
+    assert after["reshard_calls"] - before["reshard_calls"] == 1
+    assert after["kernel_launches"] - before["kernel_launches"] <= 2
+
+
+def test_config4_full_size_round_trip_and_samples(ctx):
+    """10.7 GB of traffic: checked through size-independent properties (the
+    A->B->A round trip restores every source byte; per-array XOR checksums are
+    preserved) plus exact comparison with the oracle for a sample of arrays."""
+    say("config 4 full size")
+    arrays = workloads.config(4)
+    rng = np.random.Generator(np.random.PCG64(4))
+    gs = []
+    pool = rng.standard_normal(size=1 << 24, dtype=np.float32) * np.float32(0.02)
+    for i, a in enumerate(arrays):
+        n = int(np.prod(a["shape"]))
+        reps = -(-n // pool.size)
+        g = np.tile(np.roll(pool, i * 977), reps)[:n].reshape(a["shape"]).view(np.uint32)
+        gs.append(g)
+    outs, srcs, dsts = gpu_reshard(ctx, arrays, gs, batch=True, keep=True)
+    sample = [i for i, a in enumerate(arrays) if a["name"] in
+              ("layer00.ln1", "layer00.wq", "layer11.w_in", "layer23.w_out", "embed", "final_ln", "lm_head")]
+    _compare([arrays[i] for i in sample], [gs[i] for i in sample], [outs[i] for i in sample])
+    for a, g, out in zip(arrays, gs, outs):
+        x = np.bitwise_xor.reduce(g.reshape(-1))
+        y = np.uint32(0)
+        for buf in out.values():
+            y ^= np.bitwise_xor.reduce(buf.view(np.uint32))
+        assert x == y, a["name"]
+    del outs
+    # round trip back into fresh stores laid out like the sources
+    back = [ctx.CreateStore(lib_shape(a["type"], a["src"]), name=a["name"] + ".back") for a in arrays]
+    ctx.ReshardBatch(dsts, back)
+    ctx.Sync()
+    for a, s, b in zip(arrays, srcs, back):
+        for dev in s.devices:
+            assert ctx.ReadShard(s, dev).tobytes() == ctx.ReadShard(b, dev).tobytes(), (a["name"], dev)
+    for st in srcs + dsts + back:
+        ctx.Free(st)
+
+
+def _random_array(rnd, types=("U8", "BF16", "F32", "F64", "C128")):
+    rank = rnd.randint(1, 4)
+    shape = [rnd.choice([1, 2, 3, 5, 8, 17, 33, 64, 130]) for _ in range(rank)]
+    type_ = rnd.choice(types)
+
+    def side(start):
+        shard = [rnd.randint(1, 4) for _ in range(rank)]
+        repl = rnd.choice([1, 1, 2, 3])
+        if repl == 1 and shape[-1] == 1:
+            shard[-1] = 1
+        entries = shard + ([repl] if repl > 1 else [])
+        perm = list(range(len(entries)))
+        rnd.shuffle(perm)
+        dims = [(shape[i], shard[i], perm[i]) for i in range(rank)]
+        if repl > 1:
+            dims.append((1, repl, perm[rank]))
+        d = {"dims": dims, "dev_start": start, "dev_count": int(np.prod(entries))}
+        if rnd.random() < 0.5:
+            m2m = list(range(rank))
+            rnd.shuffle(m2m)
+            d["minor_to_major"] = m2m
+        return d
+
+    return {"name": "r", "type": type_, "shape": tuple(shape), "src": side(rnd.randint(0, 3)),
+            "dst": side(rnd.randint(0, 50)), "seed": 0, "dist": "raw"}
+
+
+def test_random_sharding_pairs(ctx):
+    """Ragged extents, permuted device orders, replication on either side,
+    permuted layouts (copy, generic and transpose kernels), every element size."""
+    rnd = random.Random(1234)
+    rng = np.random.Generator(np.random.PCG64(99))
+    for case in range(60):
+        a = _random_array(rnd)
+        say("random case %d: %s %s src=%s dst=%s" % (case, a["type"], a["shape"], a["src"], a["dst"]))
+        item = ro.ITEMSIZE[a["type"]]
+        g = rng.integers(0, 256, size=int(np.prod(a["shape"])) * item, dtype=np.uint8).view(
+            ro.raw_dtype(a["type"])).reshape(a["shape"])
+        _compare([a], [g], gpu_reshard(ctx, [a], [g]))
+
+
+def test_random_batch_mixed_kernels(ctx):
+    rnd = random.Random(77)
+    rng = np.random.Generator(np.random.PCG64(5))
+    arrays, gs = [], []
+    for _ in range(25):
+        a = _random_array(rnd)
+        item = ro.ITEMSIZE[a["type"]]
+        arrays.append(a)
+        gs.append(rng.integers(0, 256, size=int(np.prod(a["shape"])) * item, dtype=np.uint8).view(
+            ro.raw_dtype(a["type"])).reshape(a["shape"]))
+    say("random batch of 25 arrays")
+    _compare(arrays, gs, gpu_reshard(ctx, arrays, gs, batch=True))
+
+
+@pytest.mark.parametrize("type_", ["U8", "BF16", "F32", "F64", "C128"])
+def test_transpose_kernel_large(ctx, type_):
+    """A minor-changing layout at a size that fills many 64x64 tiles (the LDS path)."""
+    say("transpose " + type_)
+    shape = (3, 515, 389)
+    item = ro.ITEMSIZE[type_]
+    a = {"name": "t", "type": type_, "shape": shape,
+         "src": {"dims": [(3, 1, 0), (515, 2, 1), (389, 1, 2)], "dev_start": 0, "dev_count": 2},
+         "dst": {"dims": [(3, 1, 0), (515, 1, 1), (389, 3, 2)], "dev_start": 2, "dev_count": 3,
+                 "minor_to_major": [1, 2, 0]},
+         "seed": 0, "dist": "raw"}
+    rng = np.random.Generator(np.random.PCG64(8))
+    g = rng.integers(0, 256, size=int(np.prod(shape)) * item, dtype=np.uint8).view(ro.raw_dtype(type_)).reshape(shape)
+    plan = mm.Plan(lib_shape(type_, a["src"]), lib_shape(type_, a["dst"]))
+    assert plan.stats["n_transpose_chunks"] > 0
+    _compare([a], [g], gpu_reshard(ctx, [a], [g]))
+
+
+def test_python_test_toy_shapes(ctx):
+    """The shapes the reference's end-to-end Python tests reshard: (4,4) and (8,4)
+    f32 between two 2-device meshes and from 4 devices onto 2+2."""
+    rng = np.random.Generator(np.random.PCG64(21))
+    cases = [
+        ((4, 4), [(4, 2, 0), (4, 1, 1)], (0, 2), [(4, 2, 0), (4, 1, 1)], (2, 2)),
+        ((8, 4), [(8, 2, 0), (4, 1, 1)], (0, 2), [(8, 1, 0), (4, 2, 1)], (2, 2)),
+        ((8, 4), [(8, 4, 0), (4, 1, 1)], (0, 4), [(8, 2, 0), (4, 1, 1)], (4, 2)),
+        ((8, 4), [(8, 4, 0), (4, 1, 1)], (0, 4), [(8, 1, 0), (4, 1, 1), (1, 2, 2)], (6, 2)),
+    ]
+    for shape, sd, (ss, sc), dd, (ds, dc) in cases:
+        a = {"name": "toy", "type": "F32", "shape": shape,
+             "src": {"dims": sd, "dev_start": ss, "dev_count": sc},
+             "dst": {"dims": dd, "dev_start": ds, "dev_count": dc}, "seed": 0, "dist": "raw"}
+        g = rng.standard_normal(size=shape, dtype=np.float32).view(np.uint32)
+        _compare([a], [g], gpu_reshard(ctx, [a], [g]))
+
+
+def test_scalar_broadcast_to_all_devices(ctx):
+    """mpmd_insert_reshard.cc:194-214: a scalar root output living on a 4-device
+    submesh is blasted out to all 8 devices."""
+    a = {"name": "loss", "type": "F32", "shape": (),
+         "src": {"dims": [(1, 4, 0)], "dev_start": 4, "dev_count": 4},
+         "dst": {"dims": [(1, 8, 0)], "dev_start": 0, "dev_count": 8}, "seed": 0, "dist": "raw"}
+    g = np.array(0x40490FDB, dtype=np.uint32).reshape(())
+    outs = gpu_reshard(ctx, [a], [g])
+    assert all(buf.view(np.uint32)[0] == 0x40490FDB for buf in outs[0].values())
+    assert len(outs[0]) == 8
+
+
+def test_cpu_restatement_agrees_at_full_size(ctx):
+    """Third witness at the headline size: GPU == C restatement == NumPy oracle."""
+    say("config 2 full size against the C restatement")
+    a = workloads.config(2)[0]
+    g = workloads.generate(a)
+    so, do = oracle_shape(a["type"], a["src"]), oracle_shape(a["type"], a["dst"])
+    shards = ro.make_shards(raw_global(a, g), so)
+    cpu = {d: np.empty(int(np.prod(ro.shard_shape(do))), dtype=np.uint16) for d in range(8, 12)}
+    reshard_cpu.reshard(shards, so, do, cpu, nthreads=8)
+    outs = gpu_reshard(ctx, [a], [g])
+    for dev in cpu:
+        assert outs[0][dev].tobytes() == cpu[dev].tobytes()
+
+
+def test_store_interface(ctx):
+    """CreateStore / AssembleShards / SliceLocalShard / HasLocalShard /
+    GetStoreShardedShape / Free with cache, as zuku_execute_context.h:38-133 lays them out."""
+    import torch
+    shape = mm.sharded_shape("F32", [(16, 4, 0), (8, 1, 1)], 4, 4)
+    st = ctx.CreateStore(shape, name="acts")
+    assert st.name == "acts" and st.unique_id >= 0
+    assert ctx.HasLocalShard(st, 4) and ctx.HasLocalShard(st, 7)
+    assert not ctx.HasLocalShard(st, 3) and not ctx.HasLocalShard(st, 8)
+    assert mm.describe(ctx.GetStoreShardedShape(st)) == mm.describe(shape)
+    assert st.shard_bytes == 4 * 8 * 4
+    # fresh stores are zero-filled
+    assert not ctx.ReadShard(st, 5).any()
+    # host shard in, device pointer out (zero copy view through torch)
+    data = np.arange(32, dtype=np.float32)
+    ctx.AssembleShards(shape, 6, data, existing_store=st)
+    assert ctx.ReadShard(st, 6, np.float32).tolist() == data.tolist()
+    ptr = ctx.SliceLocalShard(6, st)
+    assert ptr != 0 and ptr % 256 == 0
+    # device shard in (the GPU branch of AssembleShardsImpl): D2D from a torch tensor
+    t = torch.arange(32, dtype=torch.float32, device="cuda:0") * 2
+    torch.cuda.synchronize()
+    ctx.AssembleShards(shape, 7, t.data_ptr(), existing_store=st, size=t.numel() * 4)
+    ctx.Sync()
+    assert ctx.ReadShard(st, 7, np.float32).tolist() == (data * 2).tolist()
+    # a device outside the store's device list holds no shard
+    with pytest.raises(mm.MmrError) as e:
+        ctx.SliceLocalShard(3, st)
+    assert e.value.status_name == "NOT_FOUND"
+    with pytest.raises(mm.MmrError):
+        ctx.AssembleShards(shape, 4, np.zeros(33, dtype=np.float32), existing_store=st)  # too large
+    # Free(keep_in_cache) + CreateStore(allocate_from_cache) reuse the buffers
+    before = ctx.stats
+    ctx.Free(st, keep_in_cache=True)
+    st2 = ctx.CreateStore(shape, name="acts2", allocate_from_cache=True)
+    after = ctx.stats
+    assert after["cache_hits"] == before["cache_hits"] + 1
+    assert after["bytes_allocated"] == before["bytes_allocated"]
+    assert st2.unique_id > st.unique_id
+    ctx.Free(st2, keep_in_cache=True)
+    ctx.ClearStoreCache()
+    assert ctx.stats["bytes_allocated"] == before["bytes_allocated"] - 4 * 4096
+
+
+def test_plan_and_binding_caches(ctx):
+    """One plan per descriptor pair (keyed like ReshardKey), one pointer table per store pair."""
+    s_shape = mm.sharded_shape("BF16", [(64, 1, 0), (256, 4, 1)], 0, 4)
+    d_shape = mm.sharded_shape("BF16", [(64, 2, 0), (256, 1, 1)], 4, 2)
+    a, b = ctx.CreateStore(s_shape), ctx.CreateStore(d_shape)
+    c, d = ctx.CreateStore(s_shape), ctx.CreateStore(d_shape)
+    s0 = ctx.stats
+    ctx.Reshard(a, b)
+    ctx.Reshard(a, b)
+    ctx.Reshard(c, d)
+    ctx.Sync()
+    s1 = ctx.stats
+    assert s1["plans_built"] - s0["plans_built"] == 1
+    assert s1["bindings_built"] - s0["bindings_built"] == 2
+    assert s1["binding_cache_hits"] - s0["binding_cache_hits"] == 1
+    assert s1["reshard_calls"] - s0["reshard_calls"] == 3
+    with pytest.raises(mm.MmrError):
+        ctx.Reshard(a, a)
+    with pytest.raises(mm.MmrError):
+        ctx.Reshard(a, ctx.CreateStore(mm.sharded_shape("BF16", [(64, 2, 0), (128, 1, 1)], 4, 2)))
+    for st in (a, b, c, d):
+        ctx.Free(st)
+
+
+def test_reshard_is_stream_ordered_after_assemble(ctx):
+    """Read-after-reshard through SliceLocalShard observes the reshard of the
+    data assembled just before it, with no explicit sync in between."""
+    a = workloads.config(1, 4)[0]
+    g = workloads.generate(a)
+    srcs, dsts = make_stores(ctx, [a], [g])
+    ctx.Reshard(srcs[0], dsts[0])
+    ctx.SliceLocalShard(dsts[0].devices[0], dsts[0])  # blocks
+    _compare([a], [g], [read_all(ctx, dsts[0])])
+    ctx.Free(srcs[0]); ctx.Free(dsts[0])
