@@ -65,15 +65,14 @@ def main():
                  "MI355X's HBM and nothing here uses a second GPU (got --gpus %d)" % args.gpus)
 
     import numpy as np
-    import torch
     import multimesh_jax_amd as mm
     from multimesh_jax_amd import workloads
     from gpu_helpers import make_stores, read_all
     from helpers import oracle_outputs
 
-    if not torch.cuda.is_available():
-        sys.exit("bench.py needs a GPU: the reshard has no CPU fallback")
-
+    # No torch in this process: PyTorch bundles its own HIP runtime and two HIP
+    # runtimes cannot both drive the GPU.  The library owns its stream and its
+    # device memory; ReshardContext raises if no GPU is present (no CPU fallback).
     arrays = workloads.config(args.config)
     gs = [workloads.generate(a) for a in arrays]
     alg_bytes = workloads.algorithmic_bytes(arrays)
@@ -104,7 +103,6 @@ def main():
     for i in range(args.warmup):
         step(i)
     ctx.Sync()
-    torch.cuda.synchronize()
     # timed region: exactly K steps, wall clock bracketed by synchronisation;
     # HIP events on the context's own stream give the kernel time inside it
     t0 = time.perf_counter()
@@ -113,7 +111,6 @@ def main():
         step(i)
     kernel_ms = ctx.StopTimer()
     ctx.Sync()
-    torch.cuda.synchronize()
     wall_s = time.perf_counter() - t0
 
     ms_per_step = wall_s * 1e3 / args.steps

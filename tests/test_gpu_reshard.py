@@ -228,7 +228,6 @@ def test_cpu_restatement_agrees_at_full_size(ctx):
 def test_store_interface(ctx):
     """CreateStore / AssembleShards / SliceLocalShard / HasLocalShard /
     GetStoreShardedShape / Free with cache, as zuku_execute_context.h:38-133 lays them out."""
-    import torch
     shape = mm.sharded_shape("F32", [(16, 4, 0), (8, 1, 1)], 4, 4)
     st = ctx.CreateStore(shape, name="acts")
     assert st.name == "acts" and st.unique_id >= 0
@@ -244,12 +243,12 @@ def test_store_interface(ctx):
     assert ctx.ReadShard(st, 6, np.float32).tolist() == data.tolist()
     ptr = ctx.SliceLocalShard(6, st)
     assert ptr != 0 and ptr % 256 == 0
-    # device shard in (the GPU branch of AssembleShardsImpl): D2D from a torch tensor
-    t = torch.arange(32, dtype=torch.float32, device="cuda:0") * 2
-    torch.cuda.synchronize()
-    ctx.AssembleShards(shape, 7, t.data_ptr(), existing_store=st, size=t.numel() * 4)
-    ctx.Sync()
+    # device shard in (the GPU branch of AssembleShardsImpl): D2D from another store's buffer
+    other = ctx.CreateStore(mm.sharded_shape("F32", [(32, 1, 0)], 0, 1), name="native")
+    ctx.AssembleShards(other.shape, 0, data * 2, existing_store=other)
+    ctx.AssembleShards(shape, 7, ctx.SliceLocalShard(0, other, wait=False), existing_store=st, size=32 * 4)
     assert ctx.ReadShard(st, 7, np.float32).tolist() == (data * 2).tolist()
+    ctx.Free(other)
     # a device outside the store's device list holds no shard
     with pytest.raises(mm.MmrError) as e:
         ctx.SliceLocalShard(3, st)
