@@ -58,6 +58,9 @@ def main():
     ap.add_argument("--sets", type=int, default=3, help="independent buffer sets rotated between steps")
     ap.add_argument("--chunk-bytes", type=int, default=0)
     ap.add_argument("--order", type=int, default=0)
+    ap.add_argument("--xcd-mode", type=int, default=0)
+    ap.add_argument("--flags", type=int, default=0, help="debug plan flags")
+    ap.add_argument("--only", type=int, default=-1, help="benchmark only array i of the configuration")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -74,12 +77,14 @@ def main():
     # runtimes cannot both drive the GPU.  The library owns its stream and its
     # device memory; ReshardContext raises if no GPU is present (no CPU fallback).
     arrays = workloads.config(args.config)
+    if args.only >= 0:
+        arrays = [arrays[args.only]]
     gs = [workloads.generate(a) for a in arrays]
     alg_bytes = workloads.algorithmic_bytes(arrays)
 
     ctx = mm.ReshardContext(0)
-    if args.chunk_bytes or args.order:
-        ctx.set_plan_options(args.chunk_bytes, args.order)
+    if args.chunk_bytes or args.order or args.xcd_mode or args.flags:
+        ctx.set_plan_options(args.chunk_bytes, args.order, args.xcd_mode, args.flags)
     sets = [make_stores(ctx, arrays, gs, poison=None) for _ in range(max(1, args.sets))]
 
     def step(i):

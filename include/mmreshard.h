@@ -173,6 +173,9 @@ typedef struct {
 typedef struct {
   uint32_t chunk_bytes; /* target bytes per copy chunk, 0 = default */
   uint32_t order;       /* 0 = default; 1 generation order, 2 by destination address, 3 by source address */
+  uint32_t xcd_mode;    /* 0 = default; 1 consecutive chunks on consecutive XCDs (hardware round-robin),
+                           2 each XCD takes a contiguous eighth of the table (neighbours share an L2) */
+  uint32_t reserved;
 } mmr_plan_options;
 
 typedef struct {

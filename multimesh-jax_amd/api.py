@@ -187,12 +187,12 @@ class Plan:
     """Copy plan of one or more (source, destination) descriptor pairs."""
 
     def __init__(self, srcs: Sequence[B.ShardedShape], dsts: Sequence[B.ShardedShape],
-                 chunk_bytes: int = 0, order: int = 0):
+                 chunk_bytes: int = 0, order: int = 0, xcd_mode: int = 0):
         if isinstance(srcs, B.ShardedShape):
             srcs, dsts = [srcs], [dsts]
         self._lib = B.load()
         self._h = C.c_void_p()
-        opt = B.PlanOptions(chunk_bytes, order)
+        opt = B.PlanOptions(chunk_bytes, order, xcd_mode, 0)
         B.check(self._lib.mmr_plan_create(_shape_array(srcs), _shape_array(dsts), len(srcs), C.byref(opt),
                                           C.byref(self._h)))
 
@@ -355,8 +355,8 @@ class ReshardContext:
         B.check(self._lib.mmr_sync(self._h))
 
     # -- measurement and inspection ----------------------------------------
-    def set_plan_options(self, chunk_bytes: int = 0, order: int = 0) -> None:
-        opt = B.PlanOptions(chunk_bytes, order)
+    def set_plan_options(self, chunk_bytes: int = 0, order: int = 0, xcd_mode: int = 0, flags: int = 0) -> None:
+        opt = B.PlanOptions(chunk_bytes, order, xcd_mode, flags)
         B.check(self._lib.mmr_context_set_plan_options(self._h, C.byref(opt)))
 
     def StartTimer(self) -> None:

@@ -10,11 +10,17 @@
 namespace mmr {
 
 // Chunks whose offsets, strides and widths are all multiples of 16 bytes.
-hipError_t launch_copy16(const mmr_copy_chunk* d_chunks, int64_t n, void* const* d_ptrs, hipStream_t stream);
+// xcd_split: false = chunk i runs as workgroup i (the hardware deals consecutive
+// workgroups round-robin over the 8 XCDs); true = each XCD takes a contiguous
+// eighth of the table, so chunks that are neighbours in the table share an L2.
+hipError_t launch_copy16(const mmr_copy_chunk* d_chunks, int64_t n, void* const* d_ptrs, bool xcd_split,
+                         hipStream_t stream);
 // Chunks of any alignment (chunk.align picks the access width).
-hipError_t launch_copy_generic(const mmr_copy_chunk* d_chunks, int64_t n, void* const* d_ptrs, hipStream_t stream);
+hipError_t launch_copy_generic(const mmr_copy_chunk* d_chunks, int64_t n, void* const* d_ptrs, bool xcd_split,
+                               hipStream_t stream);
 // LDS-staged tile transposes.
-hipError_t launch_transpose(const mmr_transpose_chunk* d_chunks, int64_t n, void* const* d_ptrs, hipStream_t stream);
+hipError_t launch_transpose(const mmr_transpose_chunk* d_chunks, int64_t n, void* const* d_ptrs, bool xcd_split,
+                            hipStream_t stream);
 
 }  // namespace mmr
 

@@ -28,7 +28,8 @@ int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 class Builder {
  public:
-  Builder(mmr_plan* plan, uint32_t chunk_bytes) : plan_(plan), chunk_bytes_(chunk_bytes) {}
+  Builder(mmr_plan* plan, uint32_t chunk_bytes, bool force_generic)
+      : plan_(plan), chunk_bytes_(chunk_bytes), force_generic_(force_generic) {}
 
   void add_box(uint32_t src_slot, uint32_t dst_slot, int64_t src_off, int64_t dst_off, const BoxDim* in, int rank,
                int itemsize) {
@@ -127,12 +128,18 @@ class Builder {
                     static_cast<uint64_t>(c.s2) | static_cast<uint64_t>(c.d2);
     c.align = (bits & 15u) ? static_cast<uint32_t>(bits & (~bits + 1)) : 16u;
     if (fill) plan_->stats.n_fill_chunks += 1;
-    (c.align == 16 ? plan_->copy16 : plan_->generic).push_back(c);
+    (c.align == 16 && !force_generic_ ? plan_->copy16 : plan_->generic).push_back(c);
   }
 
   void lower_copy(uint32_t src_slot, uint32_t dst_slot, int64_t so, int64_t dof, std::vector<BoxDim>& outer, int64_t w,
                   bool fill) {
-    const int64_t cb = chunk_bytes_;
+    // Rows that are not 16-byte aligned on both sides go to the generic kernel,
+    // which spends one lane per 16-byte slot plus ragged ends: give it half the
+    // bytes per workgroup so its workgroups live about as long as aligned ones.
+    uint64_t bits = static_cast<uint64_t>(so | dof | w);
+    for (const BoxDim& d : outer) bits |= static_cast<uint64_t>(d.s | d.d);
+    const bool aligned = (bits & 15u) == 0 && !force_generic_;
+    const int64_t cb = aligned ? chunk_bytes_ : std::max<int64_t>(chunk_bytes_ / 2, 256);
     if (w > cb) {
       // long rows: split columns into near-equal segments on 256-byte boundaries of the row
       const int64_t nseg = ceil_div(w, cb);
@@ -216,6 +223,7 @@ class Builder {
 
   mmr_plan* plan_;
   uint32_t chunk_bytes_;
+  bool force_generic_;
 };
 
 int plan_one_array(Builder& b, const Side& S, const Side& D, uint32_t slot_base) {
@@ -293,9 +301,9 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
                mmr_plan* plan) {
   if (n < 0 || (n > 0 && (!srcs || !dsts))) return fail(MMR_INVALID_ARGUMENT, "bad descriptor arrays");
   uint32_t chunk_bytes = options.chunk_bytes ? options.chunk_bytes : kDefaultChunkBytes;
-  chunk_bytes = std::min<uint32_t>(std::max<uint32_t>(chunk_bytes, 1024), 16u << 20) & ~255u;
+  chunk_bytes = std::min<uint32_t>(std::max<uint32_t>(chunk_bytes, 256), 16u << 20) & ~255u;
   plan->options = options;
-  Builder builder(plan, chunk_bytes);
+  Builder builder(plan, chunk_bytes, (options.reserved & 1u) != 0);
   for (int a = 0; a < n; ++a) {
     Side S, D;
     if (int rc = make_side(srcs[a], &S)) return rc;

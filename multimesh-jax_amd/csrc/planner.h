@@ -25,7 +25,7 @@ struct mmr_plan {
 
 namespace mmr {
 
-constexpr uint32_t kDefaultChunkBytes = 64 * 1024;
+constexpr uint32_t kDefaultChunkBytes = 8 * 1024;
 constexpr uint32_t kTransposeTile = 64;  // elements per tile edge (32 for 16-byte elements)
 
 // Cache key of a batch of descriptor pairs under given options.

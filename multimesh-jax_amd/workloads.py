@@ -42,6 +42,9 @@ def config(index: int, scale: int = 1) -> List[dict]:
     """Arrays of benchmark configuration `index` (1..5).  scale > 1 divides the
     large extents so the same sharding structure runs in seconds on a CPU."""
     s = scale
+    if index == 0:  # calibration: one device to one device, i.e. a plain copy of known size (512 MiB)
+        shape = (8, 4096 // s, 8192 // s)
+        return [_array("copy", "BF16", shape, _side(shape, (1, 1, 1), 0), _side(shape, (1, 1, 1), 1), 2, "normal")]
     if index == 1:  # fp32 [4096,4096]: rows 4-way on devices 0-3 -> 2x2 blocks on devices 4-7
         shape = (4096 // s, 4096 // s)
         return [_array("c1", "F32", shape, _side(shape, (4, 1), 0), _side(shape, (2, 2), 4), 1, "uniform")]
@@ -89,6 +92,12 @@ def config(index: int, scale: int = 1) -> List[dict]:
             _array("c5b_tokens", "S32", a, _side(a, (3, 1), 0), _side(a, (5, 1), 3), 5, "int32000"),
             _array("c5b_fp8", "F8E4M3FN", b, _side(b, (3, 1), 0), _side(b, (5, 1), 3), 6, "fp8"),
         ]
+    if index == 7:  # probe: 4-byte elements, uneven 3-way -> 5-way (dword-aligned, not 16-byte-aligned runs)
+        b = (11008 // s, 1025)
+        return [_array("probe_s32", "S32", b, _side(b, (1, 3), 0), _side(b, (1, 5), 3), 7, "raw")]
+    if index == 8:  # probe: 2-byte elements, uneven 3-way -> 5-way
+        b = (11008 // s, 2051)
+        return [_array("probe_u16", "U16", b, _side(b, (1, 3), 0), _side(b, (1, 5), 3), 8, "raw")]
     raise ValueError("configuration %r" % (index,))
 
 
@@ -123,6 +132,9 @@ def generate(a: dict) -> np.ndarray:
         x = rng.standard_normal(size=shape, dtype=np.float32)
     elif dist == "normal_002":
         x = rng.standard_normal(size=shape, dtype=np.float32) * np.float32(0.02)
+    elif dist == "raw":
+        n = int(np.prod(shape)) * ITEMSIZE[a["type"]]
+        return rng.integers(0, 256, size=n, dtype=np.uint8).view("<u%d" % ITEMSIZE[a["type"]]).reshape(shape)
     elif dist == "int32000":
         return rng.integers(0, 32000, size=shape, dtype=np.int32).view(np.uint32)
     elif dist == "fp8":
