@@ -8,6 +8,6 @@ hipcc --offload-arch=gfx950 -O3 -std=c++17 -fPIC -shared \
   -Wall -Wextra -Wno-unused-command-line-argument \
   -I"${here}/../../include" -I"${here}" \
   "${here}/geometry.cc" "${here}/sharding_frontend.cc" "${here}/planner.cc" \
-  "${here}/context.cc" "${here}/kernels.hip" \
+  "${here}/context.cc" "${here}/hip_execute_context.cc" "${here}/kernels.hip" \
   -o "${out}"
 echo "built ${out}"

@@ -357,9 +357,11 @@ int mmr_store_assemble(mmr_context* ctx, mmr_store* store, int64_t device, const
   if (int rc = use_device(ctx)) return rc;
   // one flat copy of the shard's bytes, as AssembleShardsImpl does
   // (zuku_execute_context_impl.cc:405-415)
-  MMR_HIP(hipMemcpyAsync(store->base + k * store->pitch, data, size,
-                         data_on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, ctx->stream));
-  if (!data_on_device) MMR_HIP(hipStreamSynchronize(ctx->stream));  // host data is consumed before returning
+  const hipMemcpyKind kind = data_on_device == 1   ? hipMemcpyDeviceToDevice
+                             : data_on_device == 0 ? hipMemcpyHostToDevice
+                                                   : hipMemcpyDefault;  // the runtime looks the pointer up
+  MMR_HIP(hipMemcpyAsync(store->base + k * store->pitch, data, size, kind, ctx->stream));
+  if (data_on_device != 1) MMR_HIP(hipStreamSynchronize(ctx->stream));  // host data is consumed before returning
   return MMR_OK;
 }
 

@@ -1,0 +1,252 @@
+// See hip_execute_context.h.
+#include "hip_execute_context.h"
+
+#include <stdexcept>
+
+namespace mmr {
+
+namespace {
+[[noreturn]] void raise(const std::string& what) { throw std::runtime_error(what); }
+void check(int status, const char* where) {
+  if (status != MMR_OK) raise(std::string(where) + ": " + mmr_last_error());
+}
+}  // namespace
+
+mmr_sharded_shape ShardedShape::ToPod() const {
+  mmr_sharded_shape p{};
+  if (sharding.dims.size() > MMR_MAX_DIMS) raise("ShardedShape has more than MMR_MAX_DIMS entries");
+  p.dtype = static_cast<int32_t>(type);
+  p.ndims = static_cast<int32_t>(sharding.dims.size());
+  for (int i = 0; i < p.ndims; ++i)
+    p.dims[i] = mmr_sharding_dim{sharding.dims[i].size, sharding.dims[i].sharding, sharding.dims[i].permutation};
+  p.dev_start = sharding.devices.start();
+  p.dev_count = sharding.devices.size();
+  if (!minor_to_major.empty()) {
+    p.has_layout = 1;
+    for (size_t i = 0; i < minor_to_major.size() && i < MMR_MAX_DIMS; ++i) p.minor_to_major[i] = minor_to_major[i];
+  }
+  return p;
+}
+
+ShardedShape ShardedShape::FromPod(const mmr_sharded_shape& p) {
+  ShardedShape s;
+  s.type = static_cast<SupportedType>(p.dtype);
+  for (int i = 0; i < p.ndims; ++i)
+    s.sharding.dims.push_back(ShardingDim{p.dims[i].size, p.dims[i].sharding, p.dims[i].permutation});
+  s.sharding.devices = DeviceList::Create(p.dev_start, p.dev_count);
+  if (p.has_layout) {
+    int32_t rank = 0;
+    int64_t ext[MMR_MAX_DIMS];
+    check(mmr_shard_extents(&p, ext, &rank), "ShardedShape::FromPod");
+    s.minor_to_major.assign(p.minor_to_major, p.minor_to_major + rank);
+  }
+  return s;
+}
+
+int64_t ShardSize(const ShardedShape& shape) {
+  mmr_sharded_shape p = shape.ToPod();
+  int64_t bytes = 0;
+  check(mmr_shard_bytes(&p, &bytes), "ShardSize");
+  return bytes;
+}
+
+// One sharded array; freed when the last handle of the last device lets go.
+struct HipExecuteContext::SharedStore {
+  mmr_context* ctx{nullptr};
+  std::shared_ptr<std::atomic<bool>> ctx_alive;
+  mmr_store* store{nullptr};
+  ShardedShape shape;
+  bool keep_in_cache{false};
+  ~SharedStore() {
+    // a handle may outlive its context (shutdown order); the context then took the buffers with it
+    if (store && ctx_alive && ctx_alive->load()) mmr_store_free(ctx, store, keep_in_cache ? 1 : 0);
+  }
+};
+
+struct StoreHandleImpl {
+  std::shared_ptr<HipExecuteContext::SharedStore> array;
+  std::string name;
+  int64_t local_device_id{-1};
+  int64_t global_device_id{-1};
+};
+
+std::shared_ptr<HipExecuteContext> HipExecuteContext::Create(std::set<int> local_devices, int hip_device) {
+  std::shared_ptr<HipExecuteContext> c(new HipExecuteContext());
+  if (local_devices.empty()) raise("HipExecuteContext::Create: no local devices");
+  c->local_devices_ = std::move(local_devices);
+  check(mmr_context_create(hip_device, nullptr, &c->ctx_), "HipExecuteContext::Create");
+  return c;
+}
+
+HipExecuteContext::~HipExecuteContext() {
+  in_flight_.clear();  // drops the stores still attached to half-arrived ops
+  // Handles may outlive the context (Python shutdown order in the reference,
+  // zuku_execute_context_impl.cc:64-71); their stores die with the context.
+  alive_->store(false);
+  if (ctx_) mmr_context_destroy(ctx_);
+}
+
+HipExecuteContext::ReplicatedOp& HipExecuteContext::Arrive(const char* kind, int64_t local_device_id, bool* first) {
+  if (!local_devices_.count(static_cast<int>(local_device_id)))
+    raise(std::string(kind) + ": device " + std::to_string(local_device_id) + " is not a local device");
+  const int64_t seq = next_seq_[kind][local_device_id]++;
+  auto& ops = in_flight_[kind];
+  auto it = ops.find(seq);
+  *first = it == ops.end();
+  ReplicatedOp& op = ops[seq];
+  op.arrivals += 1;
+  return op;
+}
+
+void HipExecuteContext::Leave(const char* kind, int64_t seq, const ReplicatedOp& op) {
+  if (op.arrivals == static_cast<int>(local_devices_.size())) in_flight_[kind].erase(seq);
+}
+
+StoreHandle HipExecuteContext::CreateStore(int64_t local_device_id, int64_t global_device_id, ShardedShape shape,
+                                           CreateStoreConfig config) {
+  std::lock_guard<std::mutex> lock(mu_);
+  bool first = false;
+  const int64_t seq = next_seq_["CreateStore"][local_device_id];
+  ReplicatedOp& op = Arrive("CreateStore", local_device_id, &first);
+  if (first) {
+    auto shared = std::make_shared<SharedStore>();
+    shared->ctx = ctx_;
+    shared->ctx_alive = alive_;
+    shared->shape = shape;
+    mmr_sharded_shape pod = shape.ToPod();
+    const char* name = config.name.has_value() ? config.name->c_str() : nullptr;
+    int rc = mmr_store_create(ctx_, &pod, name, config.allocate_from_cache ? MMR_STORE_FROM_CACHE : 0, &shared->store);
+    if (rc != MMR_OK) {
+      in_flight_["CreateStore"].erase(seq);
+      next_seq_["CreateStore"][local_device_id]--;
+      check(rc, "CreateStore");
+    }
+    op.store = shared;
+  } else if (!(op.store->shape == shape)) {
+    raise("CreateStore: device " + std::to_string(local_device_id) + " describes store #" + std::to_string(seq) +
+          " differently from the device that created it (control replication broken)");
+  }
+  StoreHandle handle;
+  handle.impl = std::make_shared<StoreHandleImpl>();
+  handle.impl->array = op.store;
+  handle.impl->name = config.name.value_or("anonymous");
+  handle.impl->local_device_id = local_device_id;
+  handle.impl->global_device_id = global_device_id;
+  handle.unique_id = mmr_store_id(op.store->store);
+  Leave("CreateStore", seq, op);
+  return handle;
+}
+
+StoreHandle HipExecuteContext::AssembleShards(int64_t local_device_id, int64_t global_device_id, ShardedShape shape,
+                                              Shard shard, std::optional<StoreHandle> existing_store) {
+  StoreHandle output =
+      existing_store.has_value() ? *std::move(existing_store) : CreateStore(local_device_id, global_device_id, shape);
+  std::lock_guard<std::mutex> lock(mu_);
+  // across(shape.sharding.devices).if_on(p): only a member device copies its shard
+  if (shape.sharding.devices.Contains(global_device_id)) {
+    check(mmr_store_assemble(ctx_, output.impl->array->store, global_device_id, shard.data, shard.size, 2),
+          "AssembleShards");
+  }
+  return output;
+}
+
+void HipExecuteContext::Reshard(int64_t local_device_id, int64_t global_device_id, const StoreHandle& src,
+                                const StoreHandle& dst) {
+  (void)global_device_id;
+  if (!src.impl || !dst.impl) raise("Reshard: empty store handle");
+  std::lock_guard<std::mutex> lock(mu_);
+  bool first = false;
+  const int64_t seq = next_seq_["Reshard"][local_device_id];
+  ReplicatedOp& op = Arrive("Reshard", local_device_id, &first);
+  const int64_t s = src.unique_id, d = dst.unique_id;
+  if (first) {
+    op.a = s;
+    op.b = d;
+    // the whole copy runs once, on the first arriving device's call
+    int rc = mmr_reshard(ctx_, src.impl->array->store, dst.impl->array->store);
+    if (rc != MMR_OK) {
+      in_flight_["Reshard"].erase(seq);
+      next_seq_["Reshard"][local_device_id]--;
+      check(rc, "Reshard");
+    }
+  } else if (op.a != s || op.b != d) {
+    raise("Reshard: device " + std::to_string(local_device_id) + " issues reshard #" + std::to_string(seq) +
+          " on different stores than the device that started it (control replication broken)");
+  }
+  Leave("Reshard", seq, op);
+}
+
+void* HipExecuteContext::SliceLocalShard(int64_t local_device_id, const StoreHandle& handle) {
+  (void)local_device_id;
+  if (!handle.impl) raise("SliceLocalShard: empty store handle");
+  void* ptr = nullptr;
+  check(mmr_store_shard_ptr(ctx_, handle.impl->array->store, handle.impl->global_device_id, &ptr), "SliceLocalShard");
+  return ptr;
+}
+
+void HipExecuteContext::CopyShardToHost(const StoreHandle& handle, void* host_dst, size_t size) {
+  if (!handle.impl) raise("CopyShardToHost: empty store handle");
+  check(mmr_store_read_shard(ctx_, handle.impl->array->store, handle.impl->global_device_id, host_dst, size),
+        "CopyShardToHost");
+}
+
+ShardedShape HipExecuteContext::GetStoreShardedShape(const StoreHandle& handle) {
+  if (!handle.impl) raise("GetStoreShardedShape: empty store handle");
+  return handle.impl->array->shape;
+}
+
+bool HipExecuteContext::HasLocalShard(const StoreHandle& handle) {
+  if (!handle.impl) return false;
+  return handle.impl->array->shape.sharding.devices.Contains(handle.impl->global_device_id);
+}
+
+void HipExecuteContext::Free(int64_t local_device_id, StoreHandle handle, bool keep_in_cache) {
+  (void)local_device_id;
+  if (!handle.impl) return;
+  std::lock_guard<std::mutex> lock(mu_);
+  // the buffers go (back to the cache or to the allocator) when the last handle goes
+  handle.impl->array->keep_in_cache = keep_in_cache;
+  handle.impl = nullptr;
+}
+
+void HipExecuteContext::Destroy(StoreHandle& store) { store.impl = nullptr; }
+
+void HipExecuteContext::ClearStoreCache(int64_t local_device_id) {
+  (void)local_device_id;
+  check(mmr_clear_store_cache(ctx_), "ClearStoreCache");
+}
+
+void HipExecuteContext::Rename(StoreHandle& handle, std::string name) {
+  if (handle.impl) handle.impl->name = std::move(name);
+}
+
+void HipExecuteContext::CloseWindow() {}
+
+void HipExecuteContext::RunAfterAllTasks(int64_t local_device_id, std::function<void()> on_done) {
+  (void)local_device_id;
+  check(mmr_sync(ctx_), "RunAfterAllTasks");
+  on_done();
+}
+
+void HipExecuteContext::MarkProfile(const std::string& name) { (void)name; }
+
+void HipExecuteContext::StartTimer(const std::string& name) {
+  (void)name;
+  check(mmr_timer_start(ctx_), "StartTimer");
+}
+
+void HipExecuteContext::StopTimer(const std::string& name) {
+  float ms = 0;
+  check(mmr_timer_stop(ctx_, &ms), "StopTimer");
+  timers_ms_[name] = ms;
+}
+
+double HipExecuteContext::LastTimerMilliseconds(const std::string& name) { return timers_ms_[name]; }
+
+mmr_context_stats HipExecuteContext::Stats() {
+  mmr_context_stats s{};
+  check(mmr_context_get_stats(ctx_, &s), "Stats");
+  return s;
+}
+
+}  // namespace mmr

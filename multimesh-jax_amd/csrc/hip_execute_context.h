@@ -1,0 +1,197 @@
+// C++ host-side mirror of the store/reshard subset of xla::ZukuExecuteContext
+// (reference: src/pjrt_client/zuku_execute_context.h:38-133), implemented on the
+// C ABI of mmreshard.h.  Same method names, argument order and meaning, so the
+// plugin's callers (mm_pjrt_executable.cc:391-431, 495-498, 548-561, 616-658;
+// mm_pjrt_buffer.cc:141-142, 175-183) read the same against it.
+//
+// The zuku:: types the reference signatures use are mirrored here as plain
+// structs with the fields and accessors the plugin touches (mm_sharding.cc:
+// 53-61, 345-372, 638-668; mpmd_utils.cc:151-175).
+//
+// Control replication.  The plugin drives the context SPMD-style: every local
+// device issues the same calls in the same order ("for local_device in
+// num_local_devices", mm_pjrt_executable.cc:618-619).  Here all logical devices
+// live in one GPU, so the k-th CreateStore / Reshard / Free of every device
+// refers to the same sharded array / copy; the first arriving call does the
+// work and the others attach to it.  Diverging arguments between devices are
+// an invariant violation and throw.
+//
+// Errors: the reference's methods return void and abort on invariant
+// violations (zuku_execute_context_impl.cc:271-290); the mock throws
+// std::runtime_error.  This class throws std::runtime_error carrying
+// mmr_last_error(); a caller that wants the reference's behaviour aborts.
+#ifndef MMR_CSRC_HIP_EXECUTE_CONTEXT_H_
+#define MMR_CSRC_HIP_EXECUTE_CONTEXT_H_
+
+#include <atomic>
+#include <cstdint>
+#include <functional>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <optional>
+#include <set>
+#include <string>
+#include <vector>
+
+#include "mmreshard.h"
+
+namespace mmr {
+
+// zuku::SupportedType: the fifteen types mm_sharding.cc:376-425 maps to.
+enum class SupportedType : int32_t {
+  PRED = MMR_PRED, F16 = MMR_F16, BF16 = MMR_BF16, F32 = MMR_F32, F64 = MMR_F64,
+  S8 = MMR_S8, S16 = MMR_S16, S32 = MMR_S32, S64 = MMR_S64,
+  U8 = MMR_U8, U16 = MMR_U16, U32 = MMR_U32, U64 = MMR_U64, C64 = MMR_C64, C128 = MMR_C128,
+  F8E4M3FN = MMR_F8E4M3FN, F8E5M2 = MMR_F8E5M2,  // extensions
+};
+
+// zuku::ShardingDim
+struct ShardingDim {
+  int64_t size{1};
+  int64_t sharding{1};
+  int64_t permutation{0};
+  bool operator==(const ShardingDim& o) const {
+    return size == o.size && sharding == o.sharding && permutation == o.permutation;
+  }
+};
+
+// zuku::DeviceList: a contiguous range of global device ids.
+class DeviceList {
+ public:
+  struct Range {
+    int64_t start{0};
+    int64_t num_devices{0};
+  };
+  DeviceList() = default;
+  DeviceList(Range r) : range_(r) {}  // NOLINT: the reference writes DeviceList{{.start=, .num_devices=}}
+  static DeviceList Create(int64_t start, int64_t num_devices) { return DeviceList(Range{start, num_devices}); }
+  int64_t start() const { return range_.start; }
+  int64_t stop() const { return range_.start + range_.num_devices; }
+  int64_t size() const { return range_.num_devices; }
+  int64_t operator[](int64_t i) const { return range_.start + i; }
+  bool Contains(int64_t device) const { return device >= start() && device < stop(); }
+  bool Contains(const DeviceList& o) const { return o.start() >= start() && o.stop() <= stop(); }
+  bool operator==(const DeviceList& o) const { return start() == o.start() && size() == o.size(); }
+  bool operator!=(const DeviceList& o) const { return !(*this == o); }
+
+ private:
+  Range range_;
+};
+
+// zuku::ShardedShape {type, sharding{dims, devices}}
+struct ShardedShape {
+  SupportedType type{SupportedType::F32};
+  struct Sharding {
+    std::vector<ShardingDim> dims;
+    DeviceList devices;
+  } sharding;
+  std::vector<int32_t> minor_to_major;  // extension; empty = row-major shards like the reference
+
+  bool operator==(const ShardedShape& o) const {
+    return type == o.type && sharding.dims == o.sharding.dims && sharding.devices == o.sharding.devices &&
+           minor_to_major == o.minor_to_major;
+  }
+  mmr_sharded_shape ToPod() const;
+  static ShardedShape FromPod(const mmr_sharded_shape& pod);
+};
+
+// zuku::ShardSize(shape): bytes of one shard buffer (mm_mock_mm_xla.cc:75).
+int64_t ShardSize(const ShardedShape& shape);
+
+// zuku_execute_context.h:20-30
+struct Shard {
+  const void* data;
+  int64_t local_device_id;
+  size_t size;
+};
+struct CreateStoreConfig {
+  std::optional<std::string> name{std::nullopt};
+  bool allocate_from_cache{false};
+  std::optional<int64_t> min_cache_size{std::nullopt};
+};
+
+// store_handle_fwd.h:15-19, store_handle.h:16-20
+struct StoreHandleImpl;
+struct StoreHandle {
+  std::shared_ptr<StoreHandleImpl> impl{nullptr};
+  int64_t unique_id{-1};
+};
+
+// mpmd_store.h:16-25 and mpmd_partition.h:40-43, without the XLA members.
+struct Store {
+  enum class Type { PARAM, ROOT, TEMP };
+  Type type{Type::TEMP};
+  int64_t index{-1};
+  std::string name;
+  bool scalar{false};
+  ShardedShape sharded_shape;
+};
+struct Reshard {
+  Store input;
+  Store output;
+};
+
+class HipExecuteContext {
+ public:
+  // ZukuExecuteContextImpl::Create (zuku_execute_context_impl.cc:559-577).
+  // local_devices: the logical devices this process drives (all of them here).
+  static std::shared_ptr<HipExecuteContext> Create(std::set<int> local_devices, int hip_device = 0);
+  ~HipExecuteContext();
+
+  StoreHandle CreateStore(int64_t local_device_id, int64_t global_device_id, ShardedShape shape,
+                          CreateStoreConfig config = {});
+  // Shard.data: device or host memory (the runtime tells which).
+  StoreHandle AssembleShards(int64_t local_device_id, int64_t global_device_id, ShardedShape shape, Shard shard,
+                             std::optional<StoreHandle> existing_store = std::nullopt);
+  void Reshard(int64_t local_device_id, int64_t global_device_id, const StoreHandle& src, const StoreHandle& dst);
+  void* SliceLocalShard(int64_t local_device_id, const StoreHandle& handle);
+  ShardedShape GetStoreShardedShape(const StoreHandle& handle);
+  bool HasLocalShard(const StoreHandle& handle);
+  void Free(int64_t local_device_id, StoreHandle handle, bool keep_in_cache);
+  void Destroy(StoreHandle& store);
+  void ClearStoreCache(int64_t local_device_id);
+  void Rename(StoreHandle& handle, std::string name);
+
+  void OpenWindow() {}
+  void CloseWindow();
+  void RunAfterAllTasks(int64_t local_device_id, std::function<void()> on_done);
+  void MarkProfile(const std::string& name);
+  void StartTimer(const std::string& name);
+  void StopTimer(const std::string& name);
+  std::set<int> GetLocalDevices() { return local_devices_; }
+  bool IsGpu() { return true; }
+
+  // Not part of the reference interface: inspection for tests and benchmarks.
+  mmr_context* raw() { return ctx_; }
+  // What ToLiteral does through SliceLocalShard (mm_pjrt_buffer.cc:84-95): blocking copy of the handle's shard.
+  void CopyShardToHost(const StoreHandle& handle, void* host_dst, size_t size);
+  mmr_context_stats Stats();
+  double LastTimerMilliseconds(const std::string& name);
+
+ private:
+  struct SharedStore;  // one sharded array, shared by the handles of all local devices
+  struct ReplicatedOp {
+    int64_t a{-1}, b{-1};
+    std::string what;
+    std::shared_ptr<SharedStore> store;
+    int arrivals{0};
+  };
+  HipExecuteContext() = default;
+  // k-th call of `kind` on this device -> the op all devices share
+  ReplicatedOp& Arrive(const char* kind, int64_t local_device_id, bool* first);
+  void Leave(const char* kind, int64_t seq, const ReplicatedOp& op);
+
+  mmr_context* ctx_{nullptr};
+  std::shared_ptr<std::atomic<bool>> alive_{std::make_shared<std::atomic<bool>>(true)};
+  std::set<int> local_devices_;
+  std::mutex mu_;
+  std::map<std::string, std::map<int64_t, int64_t>> next_seq_;       // kind -> device -> calls so far
+  std::map<std::string, std::map<int64_t, ReplicatedOp>> in_flight_;  // kind -> seq -> op
+  std::map<std::string, double> timers_ms_;
+  friend struct StoreHandleImpl;
+};
+
+}  // namespace mmr
+
+#endif  // MMR_CSRC_HIP_EXECUTE_CONTEXT_H_

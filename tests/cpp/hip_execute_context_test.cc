@@ -1,0 +1,188 @@
+// Drives HipExecuteContext the way MultiMeshPjRtExecutable::Execute drives the
+// reference's ZukuExecuteContext (mm_pjrt_executable.cc:391-431 parameter stores,
+// :495-498 root stores, :616-658 schedule loop, mm_pjrt_buffer.cc:84-95 read-back):
+// every local device issues every call.  Results are compared with the C
+// restatement of the reshard (oracle/reshard_cpu.c), bit for bit.
+//
+// Needs a GPU.  Prints "OK" and exits 0 on success.
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "hip_execute_context.h"
+
+extern "C" {
+// oracle/reshard_cpu.c
+struct orc_desc {
+  int32_t itemsize;
+  int32_t ndims;
+  int64_t size[9];
+  int64_t sharding[9];
+  int64_t permutation[9];
+  int64_t dev_start;
+  int64_t dev_count;
+  int32_t has_layout;
+  int32_t minor_to_major[9];
+};
+int orc_reshard(const orc_desc* src, const void* const* src_bufs, const orc_desc* dst, void* const* dst_bufs,
+                int nthreads);
+}
+
+using namespace mmr;
+
+#define EXPECT(cond)                                                              \
+  do {                                                                            \
+    if (!(cond)) {                                                                \
+      std::fprintf(stderr, "FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);      \
+      return 1;                                                                   \
+    }                                                                             \
+  } while (0)
+
+static orc_desc to_orc(const ShardedShape& s, int itemsize) {
+  orc_desc d{};
+  d.itemsize = itemsize;
+  d.ndims = static_cast<int32_t>(s.sharding.dims.size());
+  for (int i = 0; i < d.ndims; ++i) {
+    d.size[i] = s.sharding.dims[i].size;
+    d.sharding[i] = s.sharding.dims[i].sharding;
+    d.permutation[i] = s.sharding.dims[i].permutation;
+  }
+  d.dev_start = s.sharding.devices.start();
+  d.dev_count = s.sharding.devices.size();
+  return d;
+}
+
+template <class Fn>
+static bool throws(Fn&& fn, const char* needle) {
+  try {
+    fn();
+  } catch (const std::runtime_error& e) {
+    return std::strstr(e.what(), needle) != nullptr;
+  }
+  return false;
+}
+
+static int run() {
+  const int kLocal = 12;
+  std::set<int> local;
+  for (int d = 0; d < kLocal; ++d) local.insert(d);
+  auto ctx = HipExecuteContext::Create(local);
+  std::printf("context created\n");
+  std::fflush(stdout);
+
+  // bf16 [4, 64, 256]: hidden 8-way on devices 0-7 -> sequence 4-way on devices 8-11
+  ShardedShape src{SupportedType::BF16, {{{4, 1, 0}, {64, 1, 1}, {256, 8, 2}}, DeviceList::Create(0, 8)}, {}};
+  ShardedShape dst{SupportedType::BF16, {{{4, 1, 0}, {64, 4, 1}, {256, 1, 2}}, DeviceList::Create(8, 4)}, {}};
+  EXPECT(ShardSize(src) == 4 * 64 * 32 * 2);
+  EXPECT(ShardSize(dst) == 4 * 16 * 256 * 2);
+
+  // native shards of the parameter, one per source device
+  std::vector<std::vector<uint16_t>> shards(8, std::vector<uint16_t>(4 * 64 * 32));
+  uint32_t lcg = 12345;
+  for (auto& s : shards)
+    for (auto& v : s) {
+      lcg = lcg * 1664525u + 1013904223u;
+      v = static_cast<uint16_t>(lcg >> 13);
+    }
+
+  // parameter stores: every local device wraps "its" native buffer (members copy, the rest attach)
+  std::vector<StoreHandle> param(kLocal), root(kLocal);
+  for (int d = 0; d < kLocal; ++d) {
+    Shard shard{d < 8 ? shards[d].data() : nullptr, d, d < 8 ? shards[d].size() * 2 : 0};
+    param[d] = ctx->AssembleShards(d, d, src, shard);
+  }
+  for (int d = 1; d < kLocal; ++d) EXPECT(param[d].unique_id == param[0].unique_id);
+  // root store of the reshard's output, created by every local device
+  for (int d = 0; d < kLocal; ++d) root[d] = ctx->CreateStore(d, d, dst, {.name = "reshard.out"});
+  for (int d = 1; d < kLocal; ++d) EXPECT(root[d].unique_id == root[0].unique_id);
+  EXPECT(root[0].unique_id != param[0].unique_id);
+  EXPECT(ctx->Stats().stores_live == 2);
+  EXPECT(ctx->GetStoreShardedShape(root[3]) == dst);
+  for (int d = 0; d < kLocal; ++d) {
+    EXPECT(ctx->HasLocalShard(param[d]) == (d < 8));
+    EXPECT(ctx->HasLocalShard(root[d]) == (d >= 8));
+  }
+
+  // schedule loop: the Reshard op, issued by every local device
+  ctx->StartTimer("execute");
+  for (int d = 0; d < kLocal; ++d) ctx->Reshard(d, d, param[d], root[d]);
+  ctx->StopTimer("execute");
+  EXPECT(ctx->Stats().reshard_calls == 1);  // the copy ran once, not twelve times
+  EXPECT(ctx->Stats().plans_built == 1);
+
+  // expectation from the CPU restatement
+  std::vector<std::vector<uint16_t>> expect(4, std::vector<uint16_t>(4 * 16 * 256, 0xDEAD));
+  {
+    orc_desc so = to_orc(src, 2), dd = to_orc(dst, 2);
+    const void* sp[8];
+    void* dp[4];
+    for (int k = 0; k < 8; ++k) sp[k] = shards[k].data();
+    for (int k = 0; k < 4; ++k) dp[k] = expect[k].data();
+    EXPECT(orc_reshard(&so, sp, &dd, dp, 2) == 0);
+  }
+  for (int d = 8; d < kLocal; ++d) {
+    void* ptr = ctx->SliceLocalShard(d, root[d]);  // blocking, as in the reference
+    EXPECT(ptr != nullptr);
+    std::vector<uint16_t> got(expect[d - 8].size());
+    ctx->CopyShardToHost(root[d], got.data(), got.size() * 2);
+    EXPECT(std::memcmp(got.data(), expect[d - 8].data(), got.size() * 2) == 0);
+  }
+  // a device outside the store's device list has no shard to slice
+  EXPECT(throws([&] { ctx->SliceLocalShard(0, root[0]); }, "holds no shard"));
+
+  // a second execution over the same stores reuses plan and pointer table
+  for (int d = 0; d < kLocal; ++d) ctx->Reshard(d, d, param[d], root[d]);
+  EXPECT(ctx->Stats().reshard_calls == 2);
+  EXPECT(ctx->Stats().plans_built == 1);
+  EXPECT(ctx->Stats().binding_cache_hits == 1);
+
+  // control replication broken: device 1 describes the k-th store differently from device 0
+  {
+    StoreHandle a = ctx->CreateStore(0, 0, dst);
+    EXPECT(throws([&] { ctx->CreateStore(1, 1, src); }, "control replication"));
+    (void)a;
+  }
+  // ... or reshards different stores than device 0 did in the same position
+  {
+    ctx->Reshard(0, 0, param[0], root[0]);
+    EXPECT(throws([&] { ctx->Reshard(1, 1, root[1], param[1]); }, "control replication"));
+  }
+
+  // Free(keep_in_cache) + CreateStore(allocate_from_cache) on a fresh context
+  auto ctx2 = HipExecuteContext::Create({0, 1});
+  ShardedShape small{SupportedType::F32, {{{16, 2, 0}}, DeviceList::Create(0, 2)}, {}};
+  StoreHandle h0 = ctx2->CreateStore(0, 0, small), h1 = ctx2->CreateStore(1, 1, small);
+  const int64_t bytes = ctx2->Stats().bytes_allocated;
+  ctx2->Free(0, h0, /*keep_in_cache=*/true);
+  EXPECT(ctx2->Stats().stores_live == 1);  // device 1 still holds it
+  ctx2->Free(1, h1, /*keep_in_cache=*/true);
+  EXPECT(ctx2->Stats().stores_live == 0);
+  StoreHandle h2 = ctx2->CreateStore(0, 0, small, {.allocate_from_cache = true});
+  StoreHandle h3 = ctx2->CreateStore(1, 1, small, {.allocate_from_cache = true});
+  EXPECT(ctx2->Stats().cache_hits == 1);
+  EXPECT(ctx2->Stats().bytes_allocated == bytes);
+  // unsupported element type and bad descriptors surface as exceptions, not aborts
+  ShardedShape bad = small;
+  bad.sharding.dims[0].permutation = 3;
+  EXPECT(throws([&] { ctx2->CreateStore(0, 0, bad); }, "permutation"));
+  // the failed call consumed no position: both devices can go on in step
+  StoreHandle h4 = ctx2->CreateStore(0, 0, small), h5 = ctx2->CreateStore(1, 1, small);
+  EXPECT(h4.unique_id == h5.unique_id);
+  ctx2->Destroy(h2);
+  ctx2->Destroy(h3);
+
+  std::printf("OK\n");
+  return 0;
+}
+
+int main() {
+  try {
+    return run();
+  } catch (const std::exception& e) {
+    std::fprintf(stderr, "ERROR: %s\n", e.what());
+    return 2;
+  }
+}

@@ -1,0 +1,187 @@
+"""The library's descriptor front-end (C++, csrc/sharding_frontend.cc) against the
+reference's known answers (tests/golden) and against the Python oracle on random inputs."""
+import numpy as np
+import pytest
+from hypothesis import given, settings, strategies as st
+
+import multimesh_jax_amd as mm
+from oracle import sharding_oracle as so
+
+
+def _lib_op(d):
+    return mm.op_sharding(type=d.get("type", "OTHER"), tile_dims=d.get("tile_dims", []),
+                          iota_reshape_dims=d.get("iota_reshape_dims", []),
+                          iota_transpose_perm=d.get("iota_transpose_perm", []),
+                          tile_assignment_devices=d.get("tile_assignment_devices", []),
+                          replicate_on_last_tile_dim=bool(d.get("replicate_on_last_tile_dim", False)),
+                          iota_offset=int(d.get("iota_offset", 0)))
+
+
+def _oracle_op(d):
+    return so.OpSharding(type=d.get("type", "OTHER"), tile_assignment_dimensions=list(d.get("tile_dims", [])),
+                         iota_reshape_dims=list(d.get("iota_reshape_dims", [])),
+                         iota_transpose_perm=list(d.get("iota_transpose_perm", [])),
+                         tile_assignment_devices=list(d.get("tile_assignment_devices", [])),
+                         replicate_on_last_tile_dim=bool(d.get("replicate_on_last_tile_dim", False)),
+                         iota_offset=int(d.get("iota_offset", 0)))
+
+
+def _op_dict(op):
+    return {"type": mm._binding.SHARDING_TYPE_NAMES[op.type],
+            "tile_dims": [op.tile_dims[i] for i in range(op.n_tile_dims)],
+            "iota_reshape_dims": [op.iota_reshape_dims[i] for i in range(op.n_iota_dims)],
+            "iota_transpose_perm": [op.iota_transpose_perm[i] for i in range(op.n_iota_dims)],
+            "replicate_on_last_tile_dim": bool(op.replicate_on_last_tile_dim), "iota_offset": op.iota_offset}
+
+
+def _strip(d):
+    d = dict(d)
+    d.pop("minor_to_major", None)
+    return d
+
+
+def test_index_math_known_answers(golden):
+    for c in golden["index_set"]:
+        assert mm.ComputeIndexSet(c["index"], c["dims"]) == c["expect"], c["source"]
+    for c in golden["global_index"]:
+        assert mm.ComputeGlobalIndex(c["indices"], c["dims"]) == c["expect"], c["source"]
+
+
+def test_logical_to_physical_known_answers(golden):
+    for c in golden["logical_to_physical"]:
+        op = mm.LogicalToPhysicalSharding(c["axes"], tuple(c["devices"]), c["mesh"], c["list_all_devices"])
+        e = c["expect"]
+        d = _op_dict(op)
+        assert d["type"] == e["type"], c["source"]
+        if "tile_dims" in e:
+            assert d["tile_dims"] == e["tile_dims"], c["source"]
+        if "device_order" in e:
+            assert mm.TileAssignmentDevices(op) == e["device_order"], c["source"]
+        if "replicate_on_last_tile_dim" in e:
+            assert d["replicate_on_last_tile_dim"] == e["replicate_on_last_tile_dim"], c["source"]
+
+
+def test_canonicalize_known_answers(golden):
+    for c in golden["canonicalize"]:
+        op = _lib_op(c["sharding"])
+        if c["expect"].get("error"):
+            with pytest.raises(mm.MmrError) as e:
+                mm.CanonicalizeSharding(op, c["shape"], c["element_type"], c["shape_is_global"])
+            assert e.value.status_name == "INVALID_ARGUMENT"
+            continue
+        got = mm.describe(mm.CanonicalizeSharding(op, c["shape"], c["element_type"], c["shape_is_global"]))
+        assert got == c["expect"], c["source"]
+
+
+def test_replicated_descriptor_and_device_override(golden):
+    for c in golden["replicated_descriptor"]:
+        got = mm.describe(mm.XlaShapeToZukuShape(c["shape"], c["element_type"], tuple(c["devices"]), _lib_op(c["sharding"])))
+        assert got == c["expect"], c["source"]
+    op = _lib_op({"tile_dims": [4, 1], "iota_reshape_dims": [4], "iota_transpose_perm": [0]})
+    ss = mm.XlaShapeToZukuShape([4, 4], "F32", (4, 4), op)
+    assert (ss.dev_start, ss.dev_count) == (4, 4)
+    with pytest.raises(mm.MmrError):
+        mm.XlaShapeToZukuShape([4, 4], "F32", (0, 8), op)
+
+
+def test_front_end_rejects_what_the_reference_rejects():
+    op = _lib_op({"tile_dims": [4, 2, 3], "iota_reshape_dims": [6, 4], "iota_transpose_perm": [1, 0]})
+    # mm_sharding.cc:422-424: no FP8 in the reference's type map
+    with pytest.raises(mm.MmrError) as e:
+        mm.CanonicalizeSharding(op, [8, 4, 6], "F8E4M3FN", True)
+    assert e.value.status_name == "UNSUPPORTED" and "Unsupported type" in str(e.value)
+    with pytest.raises(mm.MmrError) as e:
+        mm.XlaShapeToZukuShape([8, 4, 6], "F8E5M2", (0, 24), op)
+    assert e.value.status_name == "UNSUPPORTED"
+    # mm_sharding.cc:443-449: explicit device lists must count up by one
+    bad = _lib_op({"tile_dims": [2, 2], "tile_assignment_devices": [0, 2, 1, 3]})
+    with pytest.raises(mm.MmrError):
+        mm.CanonicalizeSharding(bad, [4, 4], "F32", True)
+    ok = _lib_op({"tile_dims": [2, 2], "tile_assignment_devices": [4, 5, 6, 7]})
+    assert mm.describe(mm.CanonicalizeSharding(ok, [4, 4], "F32", True)) == {
+        "type": "F32", "dims": [[4, 2, 0], [4, 2, 1]], "dev_start": 4, "dev_count": 4}
+
+
+def test_needs_reshard_truth_table(golden):
+    for c in golden["needs_reshard"]:
+        got = mm.NeedsReshard(tuple(c["operand_devices"]), tuple(c["devices"]), _lib_op(c["operand_sharding"]),
+                              _lib_op(c["sharding"]))
+        assert got == c["expect"], c["source"]
+
+
+@given(st.data())
+@settings(max_examples=200, deadline=None)
+def test_front_end_agrees_with_the_oracle_on_random_meshes(data):
+    mesh = data.draw(st.lists(st.integers(1, 4), min_size=1, max_size=4))
+    nlog = data.draw(st.integers(0, 4))
+    assign = [[] for _ in range(nlog)]
+    for ax in range(len(mesh)):
+        where = data.draw(st.integers(-1, nlog - 1))
+        if where >= 0:
+            assign[where].append(ax)
+    for a in assign:
+        data.draw(st.randoms()).shuffle(a)
+    start = data.draw(st.integers(0, 9))
+    list_all = data.draw(st.booleans())
+    count = int(np.prod(mesh))
+    lib_op = mm.LogicalToPhysicalSharding(assign, (start, count), mesh, list_all)
+    ora_op = so.logical_to_physical_sharding(assign, (start, count), mesh, list_all)
+    d = _op_dict(lib_op)
+    assert d["type"] == ora_op.type
+    if ora_op.type != "OTHER":
+        return
+    assert d["tile_dims"] == ora_op.tile_assignment_dimensions
+    assert d["iota_reshape_dims"] == ora_op.iota_reshape_dims
+    assert d["iota_transpose_perm"] == ora_op.iota_transpose_perm
+    assert d["replicate_on_last_tile_dim"] == ora_op.replicate_on_last_tile_dim
+    assert d["iota_offset"] == ora_op.iota_offset
+    assert mm.TileAssignmentDevices(lib_op) == so.iota_tile_assignment(ora_op).reshape(-1).tolist()
+    shape = [t * data.draw(st.integers(1, 3)) for t in ora_op.tile_assignment_dimensions[:nlog]]
+    is_global = data.draw(st.booleans())
+    try:
+        expect = so.canonicalize_sharding(ora_op, shape, "S32", is_global)
+    except so.ShardingError:
+        with pytest.raises(mm.MmrError):
+            mm.CanonicalizeSharding(lib_op, shape, "S32", is_global)
+        return
+    got = mm.describe(mm.CanonicalizeSharding(lib_op, shape, "S32", is_global))
+    assert got == {"type": expect.type, "dims": [[x.size, x.sharding, x.permutation] for x in expect.dims],
+                   "dev_start": expect.dev_start, "dev_count": expect.dev_count}
+    # geometry helpers agree with the oracle's device <-> tile map
+    from oracle import reshard_oracle as ro
+    ss = mm.CanonicalizeSharding(lib_op, shape, "S32", is_global)
+    for dev in range(expect.dev_start, expect.dev_start + expect.dev_count):
+        coord = ro.tile_of_device(expect, dev)
+        assert mm.tile_of_device(ss, dev) == coord
+        assert mm.device_of_tile(ss, coord) == dev
+    assert mm.shard_extents(ss) == ro.shard_shape(expect)
+
+
+@given(st.lists(st.integers(1, 4), min_size=1, max_size=4), st.data())
+@settings(max_examples=100, deadline=None)
+def test_raw_iota_shardings_agree_with_the_oracle(reshape_dims, data):
+    """Arbitrary iota reshape/transpose (not only what LogicalToPhysicalSharding emits)."""
+    perm = data.draw(st.permutations(list(range(len(reshape_dims)))))
+    n = int(np.prod(reshape_dims))
+    # tile dims: regroup the transposed iota dims into 1..3 tile dims
+    tdims = [reshape_dims[p] for p in perm]
+    cut = sorted(data.draw(st.sets(st.integers(1, max(1, len(tdims) - 1)), max_size=2))) if len(tdims) > 1 else []
+    groups, prev = [], 0
+    for c in cut + [len(tdims)]:
+        if c > prev:
+            groups.append(int(np.prod(tdims[prev:c])))
+            prev = c
+    d = {"tile_dims": groups, "iota_reshape_dims": reshape_dims, "iota_transpose_perm": list(perm),
+         "iota_offset": data.draw(st.integers(0, 5))}
+    lib_op, ora_op = _lib_op(d), _oracle_op(d)
+    assert mm.TileAssignmentDevices(lib_op) == so.iota_tile_assignment(ora_op).reshape(-1).tolist()
+    shape = [g * 2 for g in groups]
+    try:
+        expect = so.canonicalize_sharding(ora_op, shape, "F32", True)
+    except so.ShardingError:
+        with pytest.raises(mm.MmrError):
+            mm.CanonicalizeSharding(lib_op, shape, "F32", True)
+        return
+    got = mm.describe(mm.CanonicalizeSharding(lib_op, shape, "F32", True))
+    assert got["dims"] == [[x.size, x.sharding, x.permutation] for x in expect.dims]
+    assert n == got["dev_count"]
