@@ -7,6 +7,7 @@ namespace mmr {
 
 namespace {
 [[noreturn]] void raise(const std::string& what) { throw std::runtime_error(what); }
+void require_live(const StoreHandle& h, const char* where);
 void check(int status, const char* where) {
   if (status != MMR_OK) raise(std::string(where) + ": " + mmr_last_error());
 }
@@ -69,6 +70,13 @@ struct StoreHandleImpl {
   int64_t local_device_id{-1};
   int64_t global_device_id{-1};
 };
+
+namespace {
+void require_live(const StoreHandle& h, const char* where) {
+  if (!h.impl) raise(std::string(where) + ": empty store handle");
+  if (!h.impl->array) raise(std::string(where) + ": store " + std::to_string(h.unique_id) + " was freed");
+}
+}  // namespace
 
 std::shared_ptr<HipExecuteContext> HipExecuteContext::Create(std::set<int> local_devices, int hip_device) {
   std::shared_ptr<HipExecuteContext> c(new HipExecuteContext());
@@ -141,6 +149,7 @@ StoreHandle HipExecuteContext::AssembleShards(int64_t local_device_id, int64_t g
                                               Shard shard, std::optional<StoreHandle> existing_store) {
   StoreHandle output =
       existing_store.has_value() ? *std::move(existing_store) : CreateStore(local_device_id, global_device_id, shape);
+  require_live(output, "AssembleShards");
   std::lock_guard<std::mutex> lock(mu_);
   // across(shape.sharding.devices).if_on(p): only a member device copies its shard
   if (shape.sharding.devices.Contains(global_device_id)) {
@@ -153,7 +162,8 @@ StoreHandle HipExecuteContext::AssembleShards(int64_t local_device_id, int64_t g
 void HipExecuteContext::Reshard(int64_t local_device_id, int64_t global_device_id, const StoreHandle& src,
                                 const StoreHandle& dst) {
   (void)global_device_id;
-  if (!src.impl || !dst.impl) raise("Reshard: empty store handle");
+  require_live(src, "Reshard");
+  require_live(dst, "Reshard");
   std::lock_guard<std::mutex> lock(mu_);
   bool first = false;
   const int64_t seq = next_seq_["Reshard"][local_device_id];
@@ -178,25 +188,25 @@ void HipExecuteContext::Reshard(int64_t local_device_id, int64_t global_device_i
 
 void* HipExecuteContext::SliceLocalShard(int64_t local_device_id, const StoreHandle& handle) {
   (void)local_device_id;
-  if (!handle.impl) raise("SliceLocalShard: empty store handle");
+  require_live(handle, "SliceLocalShard");
   void* ptr = nullptr;
   check(mmr_store_shard_ptr(ctx_, handle.impl->array->store, handle.impl->global_device_id, &ptr), "SliceLocalShard");
   return ptr;
 }
 
 void HipExecuteContext::CopyShardToHost(const StoreHandle& handle, void* host_dst, size_t size) {
-  if (!handle.impl) raise("CopyShardToHost: empty store handle");
+  require_live(handle, "CopyShardToHost");
   check(mmr_store_read_shard(ctx_, handle.impl->array->store, handle.impl->global_device_id, host_dst, size),
         "CopyShardToHost");
 }
 
 ShardedShape HipExecuteContext::GetStoreShardedShape(const StoreHandle& handle) {
-  if (!handle.impl) raise("GetStoreShardedShape: empty store handle");
+  require_live(handle, "GetStoreShardedShape");
   return handle.impl->array->shape;
 }
 
 bool HipExecuteContext::HasLocalShard(const StoreHandle& handle) {
-  if (!handle.impl) return false;
+  if (!handle.impl || !handle.impl->array) return false;
   return handle.impl->array->shape.sharding.devices.Contains(handle.impl->global_device_id);
 }
 
@@ -204,9 +214,12 @@ void HipExecuteContext::Free(int64_t local_device_id, StoreHandle handle, bool k
   (void)local_device_id;
   if (!handle.impl) return;
   std::lock_guard<std::mutex> lock(mu_);
-  // the buffers go (back to the cache or to the allocator) when the last handle goes
+  if (!handle.impl->array) return;  // already freed through another copy of this handle
+  // As in the reference (zuku_execute_context_impl.cc:509-514) the array is taken
+  // out of the shared impl, so every copy of this device's handle lets go; the
+  // buffers go back to the cache or the allocator when the last device has freed.
   handle.impl->array->keep_in_cache = keep_in_cache;
-  handle.impl = nullptr;
+  handle.impl->array.reset();
 }
 
 void HipExecuteContext::Destroy(StoreHandle& store) { store.impl = nullptr; }

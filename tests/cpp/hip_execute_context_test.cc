@@ -160,6 +160,7 @@ static int run() {
   EXPECT(ctx2->Stats().stores_live == 1);  // device 1 still holds it
   ctx2->Free(1, h1, /*keep_in_cache=*/true);
   EXPECT(ctx2->Stats().stores_live == 0);
+  EXPECT(throws([&] { ctx2->SliceLocalShard(0, h0); }, "was freed"));  // the caller's copy of the handle is dead too
   StoreHandle h2 = ctx2->CreateStore(0, 0, small, {.allocate_from_cache = true});
   StoreHandle h3 = ctx2->CreateStore(1, 1, small, {.allocate_from_cache = true});
   EXPECT(ctx2->Stats().cache_hits == 1);
