@@ -195,11 +195,13 @@ int reshard_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* d
   const DevicePlan* dp = binding->plan;
   const mmr_plan& p = dp->plan;
   const uint32_t xm = p.options.xcd_mode;
-  MMR_HIP(mmr::launch_copy16(dp->d_copy16, static_cast<int64_t>(p.copy16.size()), binding->d_ptrs, xm == 2, ctx->stream));
+  // aligned chunks: runs of 64 table neighbours per XCD measured best across the benchmark configurations
+  MMR_HIP(mmr::launch_copy16(dp->d_copy16, static_cast<int64_t>(p.copy16.size()), binding->d_ptrs, xm == 0 ? 64 : xm,
+                             ctx->stream));
   // generic chunks leave partial lines at run boundaries; neighbours merge them when they share an L2
-  MMR_HIP(mmr::launch_copy_generic(dp->d_generic, static_cast<int64_t>(p.generic.size()), binding->d_ptrs, xm != 1,
+  MMR_HIP(mmr::launch_copy_generic(dp->d_generic, static_cast<int64_t>(p.generic.size()), binding->d_ptrs, xm == 0 ? 2 : xm,
                                    ctx->stream));
-  MMR_HIP(mmr::launch_transpose(dp->d_transposes, static_cast<int64_t>(p.transposes.size()), binding->d_ptrs, xm == 2,
+  MMR_HIP(mmr::launch_transpose(dp->d_transposes, static_cast<int64_t>(p.transposes.size()), binding->d_ptrs, xm,
                                 ctx->stream));
   ctx->stats.kernel_launches += (p.copy16.empty() ? 0 : 1) + (p.generic.empty() ? 0 : 1) + (p.transposes.empty() ? 0 : 1);
   return MMR_OK;

@@ -10,16 +10,17 @@
 namespace mmr {
 
 // Chunks whose offsets, strides and widths are all multiples of 16 bytes.
-// xcd_split: false = chunk i runs as workgroup i (the hardware deals consecutive
-// workgroups round-robin over the 8 XCDs); true = each XCD takes a contiguous
-// eighth of the table, so chunks that are neighbours in the table share an L2.
-hipError_t launch_copy16(const mmr_copy_chunk* d_chunks, int64_t n, void* const* d_ptrs, bool xcd_split,
+// xcd_mode: 0/1 = chunk i runs as workgroup i (the hardware deals consecutive
+// workgroups round-robin over the 8 XCDs); 2 = each XCD takes a contiguous
+// eighth of the table; G >= 16 = runs of G consecutive chunks share an XCD (and
+// so an L2), runs dealt round-robin.
+hipError_t launch_copy16(const mmr_copy_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
                          hipStream_t stream);
 // Chunks of any alignment (chunk.align picks the access width).
-hipError_t launch_copy_generic(const mmr_copy_chunk* d_chunks, int64_t n, void* const* d_ptrs, bool xcd_split,
+hipError_t launch_copy_generic(const mmr_copy_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
                                hipStream_t stream);
 // LDS-staged tile transposes.
-hipError_t launch_transpose(const mmr_transpose_chunk* d_chunks, int64_t n, void* const* d_ptrs, bool xcd_split,
+hipError_t launch_transpose(const mmr_transpose_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
                             hipStream_t stream);
 
 }  // namespace mmr

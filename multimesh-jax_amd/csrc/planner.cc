@@ -161,7 +161,7 @@ class Builder {
     BoxDim dim2{1, 0, 0};
     int64_t n2 = 1;
     int i2 = -1;
-    if (n1 == dim1.n && rows / n1 >= 2) {
+    if (aligned && n1 == dim1.n && rows / n1 >= 2) {  // the generic kernel walks a single row dimension
       i2 = pick_row_dim(outer, i1);
       if (i2 >= 0) {
         dim2 = outer[i2];

@@ -1,6 +1,6 @@
 #!/bin/bash
 # Builds the C++ test of the ZukuExecuteContext mirror against libmmreshard.so
-# and the C restatement of the reshard.
+# and the C restatement of the reshard, and the host emulation of the kernels.
 set -euo pipefail
 here="$(cd "$(dirname "${BASH_SOURCE[0]}")" && pwd)"
 root="${here}/../.."
@@ -10,3 +10,8 @@ g++ -O2 -std=c++20 -Wall -Wextra -I"${root}/include" -I"${root}/multimesh-jax_am
   -Wl,-rpath,'$ORIGIN/../../multimesh-jax_amd' -Wl,-rpath,'$ORIGIN/../../oracle' -Wl,-rpath,/opt/rocm/lib \
   -o "${here}/hip_execute_context_test"
 echo "built ${here}/hip_execute_context_test"
+g++ -O2 -std=c++17 -Wall -Wextra -Wno-unknown-pragmas -fPIC -shared -I"${root}/include" -I"${root}/multimesh-jax_amd/csrc" \
+  "${here}/kernel_emulation.cc" -L"${root}/multimesh-jax_amd" -lmmreshard \
+  -Wl,-rpath,'$ORIGIN/../../multimesh-jax_amd' -Wl,-rpath,/opt/rocm/lib \
+  -o "${here}/libmmr_emulation.so"
+echo "built ${here}/libmmr_emulation.so"

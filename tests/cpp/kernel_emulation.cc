@@ -1,0 +1,207 @@
+// Host emulation of the GPU kernels, for tests only.
+//
+// Runs a plan's chunk tables through the SAME per-chunk routines the kernels
+// use (multimesh-jax_amd/csrc/chunk_ops.h), one call per thread id, with a
+// memory policy that checks every access: it must lie inside one of the
+// registered shard buffers, and "aligned" accesses must be aligned.  This is
+// how index arithmetic is validated on a CPU before a kernel runs on the GPU;
+// it is never a fallback of the library.
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "chunk_ops.h"
+#include "mmreshard.h"
+
+namespace {
+
+struct Range {
+  uintptr_t lo, hi;
+};
+thread_local std::vector<Range> g_ranges;
+thread_local std::string g_error;
+thread_local uint64_t g_loaded, g_stored;
+
+void violation(const char* what, uintptr_t p, size_t n) {
+  if (!g_error.empty()) return;
+  char buf[256];
+  std::snprintf(buf, sizeof(buf), "%s of %zu bytes at %#zx", what, n, static_cast<size_t>(p));
+  g_error = buf;
+}
+
+bool inside(uintptr_t p, size_t n) {
+  for (const Range& r : g_ranges)
+    if (p >= r.lo && p + n <= r.hi) return true;
+  return false;
+}
+
+struct HostMem {
+  typedef const uint8_t* cptr;
+  typedef uint8_t* ptr;
+
+  template <typename T>
+  static T get(cptr p, size_t align, const char* what) {
+    T v{};
+    const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+    if (!inside(a, sizeof(T))) {
+      violation(what, a, sizeof(T));
+      return v;
+    }
+    if (a % align) violation("misaligned aligned-load", a, sizeof(T));
+    std::memcpy(&v, p, sizeof(T));
+    g_loaded += sizeof(T);
+    return v;
+  }
+  template <typename T>
+  static void put(ptr p, T v, size_t align, const char* what) {
+    const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+    if (!inside(a, sizeof(T))) {
+      violation(what, a, sizeof(T));
+      return;
+    }
+    if (a % align) violation("misaligned aligned-store", a, sizeof(T));
+    std::memcpy(p, &v, sizeof(T));
+    g_stored += sizeof(T);
+  }
+  static mmr::V16 load16(cptr p) { return get<mmr::V16>(p, 16, "out-of-bounds load"); }
+  static mmr::V16 load16u(cptr p) { return get<mmr::V16>(p, 1, "out-of-bounds load"); }
+  static void store16(ptr p, mmr::V16 v) { put<mmr::V16>(p, v, 16, "out-of-bounds store"); }
+  template <typename T>
+  static T loadu(cptr p) { return get<T>(p, 1, "out-of-bounds load"); }
+  template <typename T>
+  static void storeu(ptr p, T v) { put<T>(p, v, 1, "out-of-bounds store"); }
+  static uintptr_t addr(ptr p) { return reinterpret_cast<uintptr_t>(p); }
+};
+
+template <typename T, int TILE>
+void run_transpose(const mmr_transpose_chunk& c, const uint8_t* src, uint8_t* dst) {
+  constexpr int kThreads = 256;
+  static thread_local T tile[TILE][TILE + 1];
+  for (uint32_t b = 0; b < c.nb; ++b) {
+    for (uint32_t tid = 0; tid < kThreads; ++tid) mmr::transpose_load<HostMem, T, TILE, kThreads>(c, src, b, tile, tid);
+    for (uint32_t tid = 0; tid < kThreads; ++tid) mmr::transpose_store<HostMem, T, TILE, kThreads>(c, dst, b, tile, tid);
+  }
+}
+
+// Visits every workgroup of the launch grid exactly like the kernels do.
+template <class Fn>
+bool for_each_chunk(int64_t n, uint32_t xcd_mode, Fn&& fn) {
+  const uint32_t group = mmr::xcd_group_of(n, xcd_mode);
+  const uint32_t grid = mmr::grid_size(n, group);
+  std::vector<uint8_t> seen(static_cast<size_t>(n), 0);
+  for (uint32_t block = 0; block < grid; ++block) {
+    const uint32_t ci = mmr::chunk_index(block, group);
+    if (ci >= n) continue;
+    if (seen[ci]++) {
+      g_error = "chunk " + std::to_string(ci) + " visited twice by the workgroup mapping";
+      return false;
+    }
+    fn(ci);
+  }
+  for (int64_t i = 0; i < n; ++i)
+    if (!seen[i]) {
+      g_error = "chunk " + std::to_string(i) + " never visited by the workgroup mapping";
+      return false;
+    }
+  return true;
+}
+
+template <int THREADS, int UNROLL>
+void run_copy16(const mmr_copy_chunk& c, const uint8_t* src, uint8_t* dst) {
+  for (uint32_t tid = 0; tid < THREADS; ++tid) mmr::copy16_chunk<HostMem, THREADS, UNROLL>(c, src, dst, tid);
+}
+template <int THREADS, int UNROLL>
+void run_generic(const mmr_copy_chunk& c, const uint8_t* src, uint8_t* dst) {
+  for (uint32_t tid = 0; tid < THREADS; ++tid) mmr::generic_chunk<HostMem, THREADS, UNROLL>(c, src, dst, tid);
+}
+
+}  // namespace
+
+extern "C" {
+
+// slot_ptrs[i] / slot_bytes[i]: host buffer standing in for the shard buffer of
+// slot i (16-byte aligned).  shape: 0 = the kernels' default (threads, unroll),
+// other values pick the alternative instantiations.  Returns 0, or -1 with a
+// message in err.
+int mmr_emulate_plan(const mmr_plan* plan, void* const* slot_ptrs, const size_t* slot_bytes, int64_t n_slots,
+                     uint32_t xcd_mode, int shape, uint64_t* bytes_loaded, uint64_t* bytes_stored, char* err,
+                     size_t err_len) {
+  g_ranges.clear();
+  g_error.clear();
+  g_loaded = g_stored = 0;
+  for (int64_t i = 0; i < n_slots; ++i) {
+    const uintptr_t p = reinterpret_cast<uintptr_t>(slot_ptrs[i]);
+    if (p % 16) g_error = "slot buffer is not 16-byte aligned";
+    g_ranges.push_back(Range{p, p + slot_bytes[i]});
+  }
+  auto base = [&](uint32_t slot, uint64_t off) { return static_cast<uint8_t*>(slot_ptrs[slot]) + off; };
+  for (int kind = 0; kind < 2 && g_error.empty(); ++kind) {
+    const int64_t n = mmr_plan_get_copy_chunks(plan, kind, nullptr, 0);
+    std::vector<mmr_copy_chunk> chunks(static_cast<size_t>(n));
+    mmr_plan_get_copy_chunks(plan, kind, chunks.data(), n);
+    const uint32_t mode = kind == 0 ? (xcd_mode == 0 ? 64 : xcd_mode) : (xcd_mode == 0 ? 2 : xcd_mode);
+    for_each_chunk(n, mode, [&](uint32_t ci) {
+      const mmr_copy_chunk& c = chunks[ci];
+      if (c.dst_slot >= n_slots || (c.src_slot != MMR_SLOT_FILL && c.src_slot >= n_slots)) {
+        g_error = "chunk names a slot outside the pointer table";
+        return;
+      }
+      uint8_t* dst = base(c.dst_slot, c.dst_off);
+      const uint8_t* src = c.src_slot == MMR_SLOT_FILL ? dst : base(c.src_slot, c.src_off);
+      if (kind == 0) {
+        if (c.align != 16) g_error = "chunk in the aligned table is not 16-byte aligned";
+        switch (shape) {
+          case 1: run_copy16<128, 4>(c, src, dst); break;
+          case 2: run_copy16<64, 8>(c, src, dst); break;
+          case 3: run_copy16<512, 2>(c, src, dst); break;
+          default: run_copy16<256, 8>(c, src, dst); break;
+        }
+      } else {
+        if (c.n2 != 1) g_error = "generic chunk with n2 != 1";
+        switch (shape) {
+          case 1: run_generic<128, 4>(c, src, dst); break;
+          case 2: run_generic<256, 1>(c, src, dst); break;
+          case 3: run_generic<256, 4>(c, src, dst); break;
+          default: run_generic<256, 2>(c, src, dst); break;
+        }
+      }
+    });
+  }
+  if (g_error.empty()) {
+    const int64_t n = mmr_plan_get_transpose_chunks(plan, nullptr, 0);
+    std::vector<mmr_transpose_chunk> chunks(static_cast<size_t>(n));
+    mmr_plan_get_transpose_chunks(plan, chunks.data(), n);
+    for_each_chunk(n, xcd_mode, [&](uint32_t ci) {
+      const mmr_transpose_chunk& c = chunks[ci];
+      if (c.dst_slot >= n_slots || c.src_slot >= n_slots) {
+        g_error = "chunk names a slot outside the pointer table";
+        return;
+      }
+      const uint8_t* src = base(c.src_slot, c.src_off);
+      uint8_t* dst = base(c.dst_slot, c.dst_off);
+      const uint32_t tile = c.itemsize == 16 ? 32 : 64;
+      if (c.nx > tile || c.ny > tile) {
+        g_error = "transpose tile larger than the LDS tile";
+        return;
+      }
+      switch (c.itemsize) {
+        case 1: run_transpose<uint8_t, 64>(c, src, dst); break;
+        case 2: run_transpose<uint16_t, 64>(c, src, dst); break;
+        case 4: run_transpose<uint32_t, 64>(c, src, dst); break;
+        case 8: run_transpose<uint64_t, 64>(c, src, dst); break;
+        default: run_transpose<mmr::V16, 32>(c, src, dst); break;
+      }
+    });
+  }
+  if (bytes_loaded) *bytes_loaded = g_loaded;
+  if (bytes_stored) *bytes_stored = g_stored;
+  if (!g_error.empty()) {
+    if (err && err_len) std::snprintf(err, err_len, "%s", g_error.c_str());
+    return -1;
+  }
+  return 0;
+}
+
+}  // extern "C"

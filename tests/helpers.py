@@ -61,8 +61,60 @@ def apply_plan(plan: "mm.Plan", buffers: Sequence[np.ndarray]) -> None:
                     dst[do:do + it] = src[so:so + it]
 
 
+_emu = None
+
+
+def emulation_lib():
+    """tests/cpp/libmmr_emulation.so: the kernels' own per-chunk code compiled for the host with bounds checks."""
+    global _emu
+    if _emu is None:
+        import ctypes as C
+        import os
+        import subprocess
+        here = os.path.dirname(os.path.abspath(__file__))
+        path = os.path.join(here, "cpp", "libmmr_emulation.so")
+        if not os.path.exists(path):
+            subprocess.check_call(["bash", os.path.join(here, "cpp", "build.sh")])
+        lib = C.CDLL(path)
+        lib.mmr_emulate_plan.restype = C.c_int
+        lib.mmr_emulate_plan.argtypes = [C.c_void_p, C.POINTER(C.c_void_p), C.POINTER(C.c_size_t), C.c_int64,
+                                         C.c_uint32, C.c_int, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64),
+                                         C.c_char_p, C.c_size_t]
+        _emu = lib
+    return _emu
+
+
+def _aligned_copy(buf: np.ndarray) -> np.ndarray:
+    """A 64-byte aligned uint8 copy of buf (device buffers are at least that aligned)."""
+    raw = np.empty(buf.size + 64, dtype=np.uint8)
+    off = (-raw.ctypes.data) % 64
+    out = raw[off:off + buf.size]
+    out[...] = buf
+    return out
+
+
+def emulate_plan(plan: "mm.Plan", buffers: Sequence[np.ndarray], xcd_mode: int = 0, shape: int = 0):
+    """Runs the plan through the kernels' per-chunk routines on the host, in
+    place on aligned copies of `buffers`, and copies the results back.
+    Raises on any out-of-bounds or misaligned access.  Returns (loaded, stored) bytes."""
+    import ctypes as C
+    lib = emulation_lib()
+    work = [_aligned_copy(b) for b in buffers]
+    ptrs = (C.c_void_p * len(work))(*[w.ctypes.data for w in work])
+    sizes = (C.c_size_t * len(work))(*[w.size for w in work])
+    err = C.create_string_buffer(512)
+    loaded, stored = C.c_uint64(), C.c_uint64()
+    rc = lib.mmr_emulate_plan(plan._h, ptrs, sizes, len(work), xcd_mode, shape, C.byref(loaded), C.byref(stored),
+                              err, 512)
+    if rc != 0:
+        raise AssertionError("kernel emulation: " + err.value.decode())
+    for b, w in zip(buffers, work):
+        b[...] = w
+    return loaded.value, stored.value
+
+
 def run_plan_on_host(arrays: Sequence[dict], globals_: Sequence[np.ndarray], chunk_bytes: int = 0,
-                     order: int = 0, poison: int = 0xA5):
+                     order: int = 0, poison: int = 0xA5, engine: str = "numpy", xcd_mode: int = 0, shape: int = 0):
     """Returns (plan, per-array dict device -> uint8 dst buffer) after interpreting
     the batch plan on host copies of the shards."""
     srcs = [lib_shape(a["type"], a["src"]) for a in arrays]
@@ -84,7 +136,10 @@ def run_plan_on_host(arrays: Sequence[dict], globals_: Sequence[np.ndarray], chu
             buffers[base + so.dev_count + k] = buf
             out[do.dev_start + k] = buf
         outs.append(out)
-    apply_plan(plan, buffers)
+    if engine == "numpy":
+        apply_plan(plan, buffers)
+    else:
+        emulate_plan(plan, buffers, xcd_mode, shape)
     return plan, outs
 
 

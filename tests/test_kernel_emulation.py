@@ -1,0 +1,94 @@
+"""The kernels' own per-chunk code (csrc/chunk_ops.h), compiled for the host with a
+bounds- and alignment-checking memory policy, against the oracle.  Catches index
+errors and out-of-bounds accesses on a CPU, before a kernel runs on the GPU."""
+import numpy as np
+import pytest
+from hypothesis import given, settings, strategies as st
+
+from multimesh_jax_amd import workloads
+
+from helpers import oracle_outputs, run_plan_on_host
+from test_planner_cpu import random_arrays
+
+
+def _check(arrays, gs, **kw):
+    plan, outs = run_plan_on_host(arrays, gs, engine="emulation", **kw)
+    for a, g, out in zip(arrays, gs, outs):
+        expect = oracle_outputs(a, g)
+        for dev in expect:
+            assert out[dev].tobytes() == expect[dev].tobytes(), (a["name"], dev)
+    return plan
+
+
+@pytest.mark.parametrize("index,scale", [(1, 16), (2, 16), (3, 8), (5, 32), (6, 32), (7, 32), (8, 32), (11, 64)])
+@pytest.mark.parametrize("shape", [0, 1, 2, 3])
+def test_configs_through_the_kernel_code(index, scale, shape):
+    arrays = workloads.config(index, scale)
+    gs = [workloads.generate(a) for a in arrays]
+    _check(arrays, gs, shape=shape)
+
+
+@pytest.mark.parametrize("xcd_mode", [1, 2, 16, 64, 1024])
+def test_every_workgroup_mapping_visits_each_chunk_once(xcd_mode):
+    for index, scale in ((2, 32), (5, 64), (4, 64)):
+        arrays = workloads.config(index, scale)
+        gs = [workloads.generate(a) for a in arrays]
+        _check(arrays, gs, xcd_mode=xcd_mode)
+
+
+@pytest.mark.parametrize("chunk_bytes", [256, 1024, 8192, 65536, 1 << 20])
+def test_chunk_sizes_wide_and_narrow_rows(chunk_bytes):
+    # rows of 2 KiB (narrower than a 256-thread workgroup's 4 KiB pass), 8 KiB and 32 KiB (wider)
+    for index, scale in ((2, 16), (1, 4), (4, 64)):
+        arrays = workloads.config(index, scale)[:12]
+        gs = [workloads.generate(a) for a in arrays]
+        _check(arrays, gs, chunk_bytes=chunk_bytes)
+
+
+def test_traffic_of_the_headline_plan_is_exactly_algorithmic():
+    from helpers import emulate_plan, lib_shape
+    import multimesh_jax_amd as mm
+    a = workloads.config(2, 8)[0]
+    plan = mm.Plan(lib_shape(a["type"], a["src"]), lib_shape(a["type"], a["dst"]))
+    n = plan.stats["bytes_moved"]
+    bufs = [np.zeros(n // 8, dtype=np.uint8) for _ in range(8)] + [np.zeros(n // 4, dtype=np.uint8) for _ in range(4)]
+    loaded, stored = emulate_plan(plan, bufs)
+    assert loaded == n and stored == n
+
+
+@given(random_arrays(), st.sampled_from([0, 256, 2048]), st.sampled_from([0, 1, 2, 3]), st.sampled_from([0, 1, 16]))
+@settings(max_examples=200, deadline=None)
+def test_random_pairs_through_the_kernel_code(a, chunk_bytes, shape, xcd_mode):
+    from oracle import reshard_oracle as ro
+    item = ro.ITEMSIZE[a["type"]]
+    rng = np.random.Generator(np.random.PCG64(17))
+    g = rng.integers(0, 256, size=int(np.prod(a["shape"])) * item, dtype=np.uint8).view(
+        ro.raw_dtype(a["type"])).reshape(a["shape"])
+    _check([a], [g], chunk_bytes=chunk_bytes, shape=shape, xcd_mode=xcd_mode)
+
+
+@st.composite
+def ragged_2d(draw):
+    """Wide ragged rows (hundreds of bytes), the shape the generic kernel is for."""
+    rows = draw(st.integers(1, 40))
+    cols = draw(st.integers(1, 1500))
+    type_ = draw(st.sampled_from(["U8", "BF16", "S32"]))
+    st_src, st_dst = draw(st.integers(1, 4)), draw(st.integers(1, 6))
+    rs, rd = draw(st.integers(1, 3)), draw(st.integers(1, 3))
+    return {"name": "rag", "type": type_, "shape": (rows, cols),
+            "src": {"dims": [(rows, rs, 0), (cols, st_src, 1)], "dev_start": 0, "dev_count": rs * st_src},
+            "dst": {"dims": [(rows, rd, 1), (cols, st_dst, 0)], "dev_start": 20, "dev_count": rd * st_dst},
+            "seed": 0, "dist": "raw"}
+
+
+@given(ragged_2d(), st.sampled_from([0, 512, 4096]), st.sampled_from([0, 1, 2, 3]))
+@settings(max_examples=150, deadline=None)
+def test_ragged_rows_through_the_kernel_code(a, chunk_bytes, shape):
+    from oracle import reshard_oracle as ro
+    item = ro.ITEMSIZE[a["type"]]
+    rng = np.random.Generator(np.random.PCG64(23))
+    g = rng.integers(0, 256, size=int(np.prod(a["shape"])) * item, dtype=np.uint8).view(
+        ro.raw_dtype(a["type"])).reshape(a["shape"])
+    if a["shape"][1] == 1 and (a["src"]["dims"][1][1] > 1 or a["dst"]["dims"][1][1] > 1):
+        return  # trailing {1, R} would read as a replication entry
+    _check([a], [g], chunk_bytes=chunk_bytes, shape=shape)
