@@ -170,12 +170,15 @@ typedef struct {
   int64_t src_bstride, dst_bstride;
 } mmr_transpose_chunk;
 
+#define MMR_PLAN_ALL_GENERIC 1u
+
 typedef struct {
   uint32_t chunk_bytes; /* target bytes per copy chunk, 0 = default */
   uint32_t order;       /* 0 = default; 1 generation order, 2 by destination address, 3 by source address */
-  uint32_t xcd_mode;    /* 0 = default; 1 consecutive chunks on consecutive XCDs (hardware round-robin),
-                           2 each XCD takes a contiguous eighth of the table (neighbours share an L2) */
-  uint32_t reserved;
+  uint32_t xcd_mode;    /* workgroup -> chunk mapping. 0 = default; 1 = chunk i is workgroup i (the hardware deals
+                           consecutive workgroups round-robin over the 8 XCDs); 2 = each XCD takes a contiguous
+                           eighth of the table; G >= 16 = runs of G table neighbours share an XCD (and its L2) */
+  uint32_t flags;       /* MMR_PLAN_ALL_GENERIC: route aligned chunks through the generic kernel too (testing) */
 } mmr_plan_options;
 
 typedef struct {

@@ -74,7 +74,7 @@ class TransposeChunk(C.Structure):
 
 class PlanOptions(C.Structure):
     _fields_ = [("chunk_bytes", C.c_uint32), ("order", C.c_uint32), ("xcd_mode", C.c_uint32),
-                ("reserved", C.c_uint32)]
+                ("flags", C.c_uint32)]
 
 
 class PlanStats(C.Structure):

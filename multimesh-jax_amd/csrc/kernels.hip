@@ -13,7 +13,6 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
-#include <cstdlib>
 
 #include "chunk_ops.h"
 #include "kernels.h"
@@ -136,28 +135,16 @@ hipError_t check_grid(int64_t n) { return (n < 0 || n > 0x7ff00000LL) ? hipError
 
 }  // namespace
 
+// Launch shapes are the measured optimum on MI355X for 8 KiB (aligned) and
+// 4 KiB (generic) chunks: 256 threads, up to 8 (aligned) or 2 (generic) 16-byte
+// accesses in flight per lane before the first store.
 hipError_t launch_copy16(const mmr_copy_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
                          hipStream_t stream) {
   if (n == 0) return hipSuccess;
   if (hipError_t e = check_grid(n)) return e;
   const uint32_t group = xcd_group_of(n, xcd_mode);
-  static const int variant = getenv("MMR_COPY16_VARIANT") ? atoi(getenv("MMR_COPY16_VARIANT")) : 0;
-  const dim3 grid(grid_size(n, group));
-  const uint32_t count = static_cast<uint32_t>(n);
-#define MMR_V(T, U) hipLaunchKernelGGL((mmr_copy16_kernel<T, U>), grid, dim3(T), 0, stream, d_chunks, count, d_ptrs, group)
-  switch (variant) {
-    case 1: MMR_V(256, 4); break;
-    case 2: MMR_V(256, 2); break;
-    case 3: MMR_V(128, 4); break;
-    case 4: MMR_V(128, 8); break;
-    case 5: MMR_V(64, 8); break;
-    case 6: MMR_V(512, 2); break;
-    case 7: MMR_V(512, 4); break;
-    case 8: MMR_V(128, 2); break;
-    case 9: MMR_V(64, 4); break;
-    default: MMR_V(256, 8); break;
-  }
-#undef MMR_V
+  hipLaunchKernelGGL((mmr_copy16_kernel<256, 8>), dim3(grid_size(n, group)), dim3(256), 0, stream, d_chunks,
+                     static_cast<uint32_t>(n), d_ptrs, group);
   return hipGetLastError();
 }
 
@@ -166,34 +153,9 @@ hipError_t launch_copy_generic(const mmr_copy_chunk* d_chunks, int64_t n, void* 
   if (n == 0) return hipSuccess;
   if (hipError_t e = check_grid(n)) return e;
   const uint32_t group = xcd_group_of(n, xcd_mode);
-  static const int variant = getenv("MMR_GENERIC_VARIANT") ? atoi(getenv("MMR_GENERIC_VARIANT")) : 0;
-  static const int nt = getenv("MMR_GENERIC_NT") ? atoi(getenv("MMR_GENERIC_NT")) : 2;
-  const dim3 grid(grid_size(n, group));
-  const uint32_t count = static_cast<uint32_t>(n);
-#define MMR_V(T, U)                                                                                                  \
-  do {                                                                                                               \
-    if (nt == 3)                                                                                                     \
-      hipLaunchKernelGGL((mmr_copy_generic_kernel<T, U, true, true>), grid, dim3(T), 0, stream, d_chunks, count,     \
-                         d_ptrs, group);                                                                             \
-    else if (nt == 1)                                                                                                \
-      hipLaunchKernelGGL((mmr_copy_generic_kernel<T, U, true, false>), grid, dim3(T), 0, stream, d_chunks, count,    \
-                         d_ptrs, group);                                                                             \
-    else if (nt == 2)                                                                                                \
-      hipLaunchKernelGGL((mmr_copy_generic_kernel<T, U, false, true>), grid, dim3(T), 0, stream, d_chunks, count,    \
-                         d_ptrs, group);                                                                             \
-    else                                                                                                             \
-      hipLaunchKernelGGL((mmr_copy_generic_kernel<T, U, false, false>), grid, dim3(T), 0, stream, d_chunks, count,   \
-                         d_ptrs, group);                                                                             \
-  } while (0)
-  switch (variant) {
-    case 1: MMR_V(256, 4); break;
-    case 2: MMR_V(256, 1); break;
-    case 3: MMR_V(128, 4); break;
-    case 4: MMR_V(128, 2); break;
-    case 5: MMR_V(256, 8); break;
-    default: MMR_V(256, 2); break;
-  }
-#undef MMR_V
+  // cacheable loads (a source line shared by two chunks is fetched once), nontemporal stores
+  hipLaunchKernelGGL((mmr_copy_generic_kernel<256, 2, false, true>), dim3(grid_size(n, group)), dim3(256), 0, stream,
+                     d_chunks, static_cast<uint32_t>(n), d_ptrs, group);
   return hipGetLastError();
 }
 

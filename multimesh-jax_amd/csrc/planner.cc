@@ -303,7 +303,7 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
   uint32_t chunk_bytes = options.chunk_bytes ? options.chunk_bytes : kDefaultChunkBytes;
   chunk_bytes = std::min<uint32_t>(std::max<uint32_t>(chunk_bytes, 256), 16u << 20) & ~255u;
   plan->options = options;
-  Builder builder(plan, chunk_bytes, (options.reserved & 1u) != 0);
+  Builder builder(plan, chunk_bytes, (options.flags & MMR_PLAN_ALL_GENERIC) != 0);
   for (int a = 0; a < n; ++a) {
     Side S, D;
     if (int rc = make_side(srcs[a], &S)) return rc;
