@@ -10,4 +10,13 @@ hipcc --offload-arch=gfx950 -O3 -std=c++17 -fPIC -shared \
   "${here}/geometry.cc" "${here}/sharding_frontend.cc" "${here}/planner.cc" \
   "${here}/context.cc" "${here}/hip_execute_context.cc" "${here}/kernels.hip" \
   -o "${out}"
+# no kernel may touch scratch memory (a lane-indexed local array would put it there and cost most of the bandwidth)
+usage="$(hipcc --offload-arch=gfx950 -O3 -std=c++17 --cuda-device-only -c -o /dev/null \
+  -Xclang -target-feature -Xclang -packed-fp32-ops -Rpass-analysis=kernel-resource-usage \
+  -I"${here}/../../include" -I"${here}" "${here}/kernels.hip" 2>&1 | grep -E "Function Name|ScratchSize|VGPRs:|Occupancy" || true)"
+echo "${usage}" | sed 's/^.*remark: /  /'
+if echo "${usage}" | grep -E "ScratchSize \[bytes/lane\]: [1-9]" >/dev/null; then
+  echo "error: a kernel uses scratch memory" >&2
+  exit 1
+fi
 echo "built ${out}"
