@@ -170,32 +170,7 @@ typedef struct {
   int64_t src_bstride, dst_bstride;
 } mmr_transpose_chunk;
 
-/* A dense run of destination rows gathered from up to four source pieces per row
- * (source tiles that meet inside a destination row, and the zero pad of a short
- * tile as a piece without a source).  Used where rows are not 16-byte aligned:
- * the destination span is cut at its own 16-byte boundaries, so every
- * destination line is written once, whole, by one workgroup.  The planner only
- * emits a span chunk when reading up to 15 bytes before and after every source
- * run stays inside the source shard buffer. */
-#define MMR_SPAN_MAX_PIECES 4
-typedef struct {
-  uint32_t src_slot; /* MMR_SLOT_FILL: zeros */
-  uint32_t w;        /* bytes of this piece in every row */
-  uint64_t src_off;  /* first row's first byte, from the slot's base */
-  int64_t s1;        /* source byte stride between rows */
-} mmr_span_piece;
-typedef struct {
-  uint32_t dst_slot;
-  uint32_t n_pieces;
-  uint64_t dst_off;   /* first byte of the span */
-  uint32_t row_bytes; /* sum of the piece widths: destination rows are back to back */
-  uint32_t n_rows;
-  uint32_t reserved0, reserved1;
-  mmr_span_piece pieces[MMR_SPAN_MAX_PIECES];
-} mmr_span_chunk;
-
 #define MMR_PLAN_ALL_GENERIC 1u
-#define MMR_PLAN_NO_SPANS 2u
 
 typedef struct {
   uint32_t chunk_bytes; /* target bytes per copy chunk, 0 = default */
@@ -203,8 +178,7 @@ typedef struct {
   uint32_t xcd_mode;    /* workgroup -> chunk mapping. 0 = default; 1 = chunk i is workgroup i (the hardware deals
                            consecutive workgroups round-robin over the 8 XCDs); 2 = each XCD takes a contiguous
                            eighth of the table; G >= 16 = runs of G table neighbours share an XCD (and its L2) */
-  uint32_t flags;       /* MMR_PLAN_ALL_GENERIC: route aligned chunks through the generic kernel too (testing);
-                           MMR_PLAN_NO_SPANS: never use span chunks (ragged rows then go row by row) */
+  uint32_t flags;       /* MMR_PLAN_ALL_GENERIC: route aligned chunks through the generic kernel too (testing) */
 } mmr_plan_options;
 
 typedef struct {
@@ -213,7 +187,6 @@ typedef struct {
   int64_t n_copy16_chunks;     /* 16-byte aligned copy chunks */
   int64_t n_copy_generic_chunks;
   int64_t n_transpose_chunks;
-  int64_t n_span_chunks;
   int64_t n_fill_chunks;       /* included in the two copy counts */
   int64_t bytes_moved;         /* valid bytes written = valid bytes read */
   int64_t bytes_filled;        /* pad bytes zeroed */
@@ -228,7 +201,6 @@ int mmr_plan_get_stats(const mmr_plan* plan, mmr_plan_stats* out);
 /* kind: 0 = 16-byte aligned copy chunks, 1 = generic copy chunks. Returns how many were written. */
 int64_t mmr_plan_get_copy_chunks(const mmr_plan* plan, int32_t kind, mmr_copy_chunk* out, int64_t capacity);
 int64_t mmr_plan_get_transpose_chunks(const mmr_plan* plan, mmr_transpose_chunk* out, int64_t capacity);
-int64_t mmr_plan_get_span_chunks(const mmr_plan* plan, mmr_span_chunk* out, int64_t capacity);
 int64_t mmr_plan_get_slot_bases(const mmr_plan* plan, int64_t* out, int64_t capacity);
 
 /* ---------------------------------------------------------------------------

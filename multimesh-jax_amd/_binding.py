@@ -72,18 +72,6 @@ class TransposeChunk(C.Structure):
     ]
 
 
-class SpanPiece(C.Structure):
-    _fields_ = [("src_slot", C.c_uint32), ("w", C.c_uint32), ("src_off", C.c_uint64), ("s1", C.c_int64)]
-
-
-class SpanChunk(C.Structure):
-    _fields_ = [
-        ("dst_slot", C.c_uint32), ("n_pieces", C.c_uint32), ("dst_off", C.c_uint64),
-        ("row_bytes", C.c_uint32), ("n_rows", C.c_uint32), ("reserved0", C.c_uint32), ("reserved1", C.c_uint32),
-        ("pieces", SpanPiece * 4),
-    ]
-
-
 class PlanOptions(C.Structure):
     _fields_ = [("chunk_bytes", C.c_uint32), ("order", C.c_uint32), ("xcd_mode", C.c_uint32),
                 ("flags", C.c_uint32)]
@@ -91,7 +79,7 @@ class PlanOptions(C.Structure):
 
 class PlanStats(C.Structure):
     _fields_ = [(n, C.c_int64) for n in (
-        "n_arrays", "n_boxes", "n_copy16_chunks", "n_copy_generic_chunks", "n_transpose_chunks", "n_span_chunks",
+        "n_arrays", "n_boxes", "n_copy16_chunks", "n_copy_generic_chunks", "n_transpose_chunks",
         "n_fill_chunks", "bytes_moved", "bytes_filled", "table_bytes", "n_slots")]
 
     def as_dict(self):
@@ -133,7 +121,6 @@ PROTOTYPES = {
     "mmr_plan_get_stats": (C.c_int, [VP, P(PlanStats)]),
     "mmr_plan_get_copy_chunks": (I64, [VP, I32, P(CopyChunk), I64]),
     "mmr_plan_get_transpose_chunks": (I64, [VP, P(TransposeChunk), I64]),
-    "mmr_plan_get_span_chunks": (I64, [VP, P(SpanChunk), I64]),
     "mmr_plan_get_slot_bases": (I64, [VP, P(I64), I64]),
     "mmr_context_create": (C.c_int, [I32, VP, P(VP)]),
     "mmr_context_destroy": (None, [VP]),

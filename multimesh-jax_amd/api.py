@@ -187,12 +187,12 @@ class Plan:
     """Copy plan of one or more (source, destination) descriptor pairs."""
 
     def __init__(self, srcs: Sequence[B.ShardedShape], dsts: Sequence[B.ShardedShape],
-                 chunk_bytes: int = 0, order: int = 0, xcd_mode: int = 0, flags: int = 0):
+                 chunk_bytes: int = 0, order: int = 0, xcd_mode: int = 0):
         if isinstance(srcs, B.ShardedShape):
             srcs, dsts = [srcs], [dsts]
         self._lib = B.load()
         self._h = C.c_void_p()
-        opt = B.PlanOptions(chunk_bytes, order, xcd_mode, flags)
+        opt = B.PlanOptions(chunk_bytes, order, xcd_mode, 0)
         B.check(self._lib.mmr_plan_create(_shape_array(srcs), _shape_array(dsts), len(srcs), C.byref(opt),
                                           C.byref(self._h)))
 
@@ -219,20 +219,6 @@ class Plan:
         buf = (B.TransposeChunk * max(n, 1))()
         self._lib.mmr_plan_get_transpose_chunks(self._h, buf, n)
         return np.frombuffer(buf, dtype=np.dtype(B.TransposeChunk), count=n).copy()
-
-    def span_chunks(self) -> list:
-        """Span chunks as plain dicts (pieces as a list of dicts)."""
-        n = self._lib.mmr_plan_get_span_chunks(self._h, None, 0)
-        buf = (B.SpanChunk * max(n, 1))()
-        self._lib.mmr_plan_get_span_chunks(self._h, buf, n)
-        out = []
-        for i in range(n):
-            c = buf[i]
-            out.append({"dst_slot": c.dst_slot, "dst_off": c.dst_off, "row_bytes": c.row_bytes, "n_rows": c.n_rows,
-                        "pieces": [{"src_slot": c.pieces[j].src_slot, "w": c.pieces[j].w,
-                                    "src_off": c.pieces[j].src_off, "s1": c.pieces[j].s1}
-                                   for j in range(c.n_pieces)]})
-        return out
 
     def slot_bases(self) -> List[int]:
         n = self._lib.mmr_plan_get_slot_bases(self._h, None, 0)

@@ -231,113 +231,6 @@ MMR_HD void generic_chunk(const mmr_copy_chunk& c, typename M::cptr src, typenam
 }
 
 // ---------------------------------------------------------------------------
-// Span: n_rows destination rows that lie back to back (row_bytes each), every
-// row gathered from up to four source pieces (and zeros for a pad piece).  The
-// span is cut at the 16-byte boundaries of the DESTINATION; a lane owns one
-// aligned slot and assembles its 16 bytes from the one, two or (rarely) three
-// source runs that meet inside it: for each run one unaligned 16-byte load
-// positioned so the wanted bytes land in place, then a byte-mask merge.  Only
-// the first and last slot of the whole span can be partial; every other store
-// is one aligned 16 bytes.  Loads may read up to 15 bytes before or after a
-// source run; the planner only builds a span where that stays in the buffer.
-// Threads step through slots tid, tid + THREADS, ...; (row, col) of a slot is
-// advanced by a precomputed quotient and remainder, no division in the loop.
-// ---------------------------------------------------------------------------
-template <class M>
-struct SpanSources {
-  typename M::cptr base[MMR_SPAN_MAX_PIECES];  // slot base + src_off of every piece (unused for fill pieces)
-};
-
-MMR_HD uint32_t low_bytes_mask(uint32_t nbytes) { return nbytes >= 4u ? 0xFFFFFFFFu : ((1u << (8u * nbytes)) - 1u); }
-
-// bytes [a, a + len) of `out` := the same bytes of `b`
-MMR_HD uint32_t merge_dword(uint32_t o, uint32_t n, uint32_t a, uint32_t e, uint32_t base) {
-  const uint32_t lo_b = a > base ? (a - base < 4u ? a - base : 4u) : 0u;
-  const uint32_t hi_b = e > base ? (e - base < 4u ? e - base : 4u) : 0u;
-  const uint32_t mask = low_bytes_mask(hi_b) & ~low_bytes_mask(lo_b);
-  return (o & ~mask) | (n & mask);
-}
-MMR_HD V16 merge_bytes(V16 out, V16 b, uint32_t a, uint32_t len) {
-  const uint32_t e = a + len;
-  return V16{merge_dword(out.x, b.x, a, e, 0u), merge_dword(out.y, b.y, a, e, 4u), merge_dword(out.z, b.z, a, e, 8u),
-             merge_dword(out.w, b.w, a, e, 12u)};
-}
-
-MMR_HD uint8_t byte_of(V16 v, uint32_t i) {
-  const uint32_t d = i < 4u ? v.x : (i < 8u ? v.y : (i < 12u ? v.z : v.w));
-  return static_cast<uint8_t>(d >> (8u * (i & 3u)));
-}
-
-template <class M, int THREADS>
-MMR_HD void span_chunk(const mmr_span_chunk& c, const SpanSources<M>& srcs, typename M::ptr dst, uint32_t tid) {
-  const uint32_t rb = c.row_bytes;
-  const int32_t total = static_cast<int32_t>(rb * c.n_rows);
-  const int32_t mis = static_cast<int32_t>(M::addr(dst) & 15u);
-  const uint32_t slots = static_cast<uint32_t>(mis + total + 15) >> 4;
-  const uint32_t stepq = (16u * THREADS) / rb, stepr = (16u * THREADS) - stepq * rb;
-  // pos: span-relative byte where this thread's aligned slot starts (negative only for slot 0);
-  // (row, col) = position of pos in the span, col signed so slot 0 needs no special case
-  int32_t pos = static_cast<int32_t>(16u * tid) - mis;
-  uint32_t row = pos > 0 ? static_cast<uint32_t>(pos) / rb : 0u;
-  int32_t col = pos - static_cast<int32_t>(row * rb);
-  for (uint32_t k = tid; k < slots; k += THREADS) {
-    const int32_t lo = pos < 0 ? 0 : pos;
-    const int32_t hi = pos + 16 < total ? pos + 16 : total;
-    V16 out{0, 0, 0, 0};
-    int32_t p = lo;
-    uint32_t r = row;
-    uint32_t cc = col < 0 ? 0u : static_cast<uint32_t>(col);
-    while (p < hi) {
-      // the piece that holds column cc; indices are compile-time constants so the
-      // piece table stays in registers (a lane-varying index would spill it to scratch)
-      uint32_t cstart = 0, pw = c.pieces[0].w, pslot = c.pieces[0].src_slot;
-      int64_t ps1 = c.pieces[0].s1;
-      typename M::cptr pbase = srcs.base[0];
-#pragma unroll
-      for (uint32_t q = 1; q < MMR_SPAN_MAX_PIECES; ++q) {
-        if (q < c.n_pieces && cc >= cstart + pw) {
-          cstart += pw;
-          pw = c.pieces[q].w;
-          pslot = c.pieces[q].src_slot;
-          ps1 = c.pieces[q].s1;
-          pbase = srcs.base[q];
-        }
-      }
-      const uint32_t left_in_piece = cstart + pw - cc;
-      const uint32_t want = static_cast<uint32_t>(hi - p);
-      const uint32_t seg = want < left_in_piece ? want : left_in_piece;
-      if (pslot != MMR_SLOT_FILL) {
-        const uint32_t a = static_cast<uint32_t>(p - pos);  // where in the slot this run lands
-        typename M::cptr sa = pbase + (r * ps1 + (cc - cstart));
-        const V16 b = M::load16u(sa - a);
-        out = seg == 16u ? b : merge_bytes(out, b, a, seg);
-      }
-      p += static_cast<int32_t>(seg);
-      cc += seg;
-      if (cc == rb) {
-        cc = 0;
-        ++r;
-      }
-    }
-    if (hi - lo == 16) {
-      M::store16(dst + pos, out);
-    } else {
-      for (int32_t i = lo; i < hi; ++i) M::template storeu<uint8_t>(dst + i, byte_of(out, static_cast<uint32_t>(i - pos)));
-    }
-    pos += 16 * THREADS;
-    row += stepq;
-    col += static_cast<int32_t>(stepr);
-    if (col >= static_cast<int32_t>(rb)) {
-      col -= static_cast<int32_t>(rb);
-      ++row;
-    } else if (col < 0) {  // only after slot 0: pos is positive from here on, so borrow from the row
-      col += static_cast<int32_t>(rb);
-      --row;
-    }
-  }
-}
-
-// ---------------------------------------------------------------------------
 // Tile transpose: x is contiguous in the source, y in the destination.  Rows of
 // the tile are read along x into tile[y][x] (row pitch TILE + 1 elements to
 // spread the column reads over the LDS banks) and written along y.  The caller

@@ -34,8 +34,6 @@ struct DevicePlan {
   mmr_copy_chunk* d_copy16 = nullptr;
   mmr_copy_chunk* d_generic = nullptr;
   mmr_transpose_chunk* d_transposes = nullptr;
-  mmr_span_chunk* d_spans = nullptr;
-  mmr::PlanTables tables{};
 };
 
 struct Binding {
@@ -135,16 +133,6 @@ int get_plan(mmr_context* ctx, const std::vector<mmr_sharded_shape>& srcs, const
   if (int rc = upload(ctx, dp->plan.copy16, &dp->d_copy16)) return rc;
   if (int rc = upload(ctx, dp->plan.generic, &dp->d_generic)) return rc;
   if (int rc = upload(ctx, dp->plan.transposes, &dp->d_transposes)) return rc;
-  if (int rc = upload(ctx, dp->plan.spans, &dp->d_spans)) return rc;
-  // Workgroup -> chunk mapping per table.  Aligned chunks and spans: runs of 64
-  // table neighbours per XCD measured best across the benchmark configurations;
-  // generic chunks leave partial lines at run boundaries, so each XCD takes a
-  // contiguous eighth of that table and neighbours merge in one L2.
-  const uint32_t xm = ctx->options.xcd_mode;
-  mmr::set_table(&dp->tables.copy16, dp->d_copy16, static_cast<int64_t>(dp->plan.copy16.size()), xm == 0 ? 64 : xm);
-  mmr::set_table(&dp->tables.span, dp->d_spans, static_cast<int64_t>(dp->plan.spans.size()), xm == 0 ? 64 : xm);
-  mmr::set_table(&dp->tables.generic, dp->d_generic, static_cast<int64_t>(dp->plan.generic.size()), xm == 0 ? 2 : xm);
-  mmr::set_table(&dp->tables.transpose, dp->d_transposes, static_cast<int64_t>(dp->plan.transposes.size()), xm);
   ctx->stats.plans_built += 1;
   *out = dp.get();
   ctx->plans.emplace(std::move(key), std::move(dp));
@@ -205,8 +193,17 @@ int reshard_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* d
     ctx->bindings.emplace(ids, std::move(b));
   }
   const DevicePlan* dp = binding->plan;
-  MMR_HIP(mmr::launch_plan(dp->tables, binding->d_ptrs, ctx->stream));
-  ctx->stats.kernel_launches += 1;
+  const mmr_plan& p = dp->plan;
+  const uint32_t xm = p.options.xcd_mode;
+  // aligned chunks: runs of 64 table neighbours per XCD measured best across the benchmark configurations
+  MMR_HIP(mmr::launch_copy16(dp->d_copy16, static_cast<int64_t>(p.copy16.size()), binding->d_ptrs, xm == 0 ? 64 : xm,
+                             ctx->stream));
+  // generic chunks leave partial lines at run boundaries; neighbours merge them when they share an L2
+  MMR_HIP(mmr::launch_copy_generic(dp->d_generic, static_cast<int64_t>(p.generic.size()), binding->d_ptrs, xm == 0 ? 2 : xm,
+                                   ctx->stream));
+  MMR_HIP(mmr::launch_transpose(dp->d_transposes, static_cast<int64_t>(p.transposes.size()), binding->d_ptrs, xm,
+                                ctx->stream));
+  ctx->stats.kernel_launches += (p.copy16.empty() ? 0 : 1) + (p.generic.empty() ? 0 : 1) + (p.transposes.empty() ? 0 : 1);
   return MMR_OK;
 }
 
@@ -255,7 +252,6 @@ void mmr_context_destroy(mmr_context* ctx) {
     (void)hipFree(p.second->d_copy16);
     (void)hipFree(p.second->d_generic);
     (void)hipFree(p.second->d_transposes);
-    (void)hipFree(p.second->d_spans);
   }
   for (auto& s : ctx->stores) (void)hipFree(s.second->base);
   for (auto& c : ctx->buffer_cache)

@@ -1,5 +1,5 @@
-// Launcher of the gfx950 data-movement kernel.  One launch consumes all chunk
-// tables of a plan: the grid is the tables back to back, one workgroup per chunk.
+// Launchers of the gfx950 data-movement kernels. One launch consumes one chunk
+// table of a plan: workgroup i executes chunk i.
 #ifndef MMR_CSRC_KERNELS_H_
 #define MMR_CSRC_KERNELS_H_
 
@@ -9,27 +9,19 @@
 
 namespace mmr {
 
-// Device-resident chunk tables of one plan, as the kernel receives them (by value).
-struct PlanTables {
-  struct Table {
-    const void* chunks;  // device pointer to the records
-    uint32_t n;          // records
-    uint32_t group;      // XCD grouping: runs of `group` table neighbours share an XCD
-    uint32_t grid;       // workgroups reserved for the table (n padded to the grouping)
-  };
-  Table copy16;     // mmr_copy_chunk, every offset/stride/width a multiple of 16
-  Table span;       // mmr_span_chunk
-  Table generic;    // mmr_copy_chunk, any alignment
-  Table transpose;  // mmr_transpose_chunk
-};
-
+// Chunks whose offsets, strides and widths are all multiples of 16 bytes.
 // xcd_mode: 0/1 = chunk i runs as workgroup i (the hardware deals consecutive
 // workgroups round-robin over the 8 XCDs); 2 = each XCD takes a contiguous
 // eighth of the table; G >= 16 = runs of G consecutive chunks share an XCD (and
 // so an L2), runs dealt round-robin.
-void set_table(PlanTables::Table* t, const void* d_chunks, int64_t n, uint32_t xcd_mode);
-
-hipError_t launch_plan(const PlanTables& tables, void* const* d_ptrs, hipStream_t stream);
+hipError_t launch_copy16(const mmr_copy_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
+                         hipStream_t stream);
+// Chunks of any alignment (chunk.align picks the access width).
+hipError_t launch_copy_generic(const mmr_copy_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
+                               hipStream_t stream);
+// LDS-staged tile transposes.
+hipError_t launch_transpose(const mmr_transpose_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
+                            hipStream_t stream);
 
 }  // namespace mmr
 

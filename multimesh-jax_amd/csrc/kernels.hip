@@ -75,56 +75,50 @@ __device__ __forceinline__ gchar* slot_base(void* const* __restrict__ ptrs, uint
   return (gchar*)(static_cast<char*>(ptrs[slot])) + off;
 }
 
-constexpr int kThreads = 256;  // every chunk class runs 256-thread workgroups (4 wavefronts)
-
-// Launch shapes are the measured optimum on MI355X for 8 KiB (aligned) and
-// 4 KiB (generic, span) chunks: up to 8 (aligned) or 2 (generic) 16-byte
-// accesses in flight per lane before the first store.
-__device__ __forceinline__ void run_copy16(const mmr_copy_chunk* __restrict__ chunks, uint32_t ci,
-                                           void* const* __restrict__ ptrs) {
+template <int THREADS, int UNROLL>
+__global__ __launch_bounds__(THREADS) void mmr_copy16_kernel(const mmr_copy_chunk* __restrict__ chunks, uint32_t n,
+                                                             void* const* __restrict__ ptrs, uint32_t xcd_group) {
+  const uint32_t ci = chunk_index(blockIdx.x, xcd_group);
+  if (ci >= n) return;
   const mmr_copy_chunk c = chunks[ci];
   gchar* dst = slot_base(ptrs, c.dst_slot, c.dst_off);
   gcchar* src = c.src_slot == MMR_SLOT_FILL ? dst : slot_base(ptrs, c.src_slot, c.src_off);  // never read when filling
-  copy16_chunk<DeviceMem<true, true>, kThreads, 8>(c, src, dst, threadIdx.x);
+  copy16_chunk<DeviceMem<true, true>, THREADS, UNROLL>(c, src, dst, threadIdx.x);
 }
 
-__device__ __forceinline__ void run_generic(const mmr_copy_chunk* __restrict__ chunks, uint32_t ci,
-                                            void* const* __restrict__ ptrs) {
+template <int THREADS, int UNROLL, bool NTL, bool NTS>
+__global__ __launch_bounds__(THREADS) void mmr_copy_generic_kernel(const mmr_copy_chunk* __restrict__ chunks, uint32_t n,
+                                                                   void* const* __restrict__ ptrs, uint32_t xcd_group) {
+  const uint32_t ci = chunk_index(blockIdx.x, xcd_group);
+  if (ci >= n) return;
   const mmr_copy_chunk c = chunks[ci];
   gchar* dst = slot_base(ptrs, c.dst_slot, c.dst_off);
-  gcchar* src = c.src_slot == MMR_SLOT_FILL ? dst : slot_base(ptrs, c.src_slot, c.src_off);
-  // cacheable loads (a source line shared by two chunks is fetched once), nontemporal stores
-  generic_chunk<DeviceMem<false, true>, kThreads, 2>(c, src, dst, threadIdx.x);
+  gcchar* src = c.src_slot == MMR_SLOT_FILL ? dst : slot_base(ptrs, c.src_slot, c.src_off);  // never read when filling
+  generic_chunk<DeviceMem<NTL, NTS>, THREADS, UNROLL>(c, src, dst, threadIdx.x);
 }
 
-__device__ __forceinline__ void run_span(const mmr_span_chunk* __restrict__ chunks, uint32_t ci,
-                                         void* const* __restrict__ ptrs) {
-  typedef DeviceMem<false, true> M;  // cacheable loads: neighbouring slots and rows share source lines
-  const mmr_span_chunk c = chunks[ci];
-  gchar* dst = slot_base(ptrs, c.dst_slot, c.dst_off);
-  SpanSources<M> srcs;
-#pragma unroll
-  for (uint32_t j = 0; j < MMR_SPAN_MAX_PIECES; ++j) {
-    const bool live = j < c.n_pieces && c.pieces[j].src_slot != MMR_SLOT_FILL;
-    srcs.base[j] = live ? slot_base(ptrs, c.pieces[j].src_slot, c.pieces[j].src_off) : dst;  // never read when not live
-  }
-  span_chunk<M, kThreads>(c, srcs, dst, threadIdx.x);
-}
+constexpr int kTransposeThreads = 256;
 
 template <typename T, int TILE>
 __device__ __forceinline__ void transpose_tiles(const mmr_transpose_chunk& c, gcchar* src, gchar* dst, void* lds_raw) {
   typedef DeviceMem<true, true> M;
   T(*tile)[TILE + 1] = reinterpret_cast<T(*)[TILE + 1]>(lds_raw);
   for (uint32_t b = 0; b < c.nb; ++b) {
-    transpose_load<M, T, TILE, kThreads>(c, src, b, tile, threadIdx.x);
+    transpose_load<M, T, TILE, kTransposeThreads>(c, src, b, tile, threadIdx.x);
     __syncthreads();
-    transpose_store<M, T, TILE, kThreads>(c, dst, b, tile, threadIdx.x);
+    transpose_store<M, T, TILE, kTransposeThreads>(c, dst, b, tile, threadIdx.x);
     __syncthreads();
   }
 }
 
-__device__ __forceinline__ void run_transpose(const mmr_transpose_chunk* __restrict__ chunks, uint32_t ci,
-                                              void* const* __restrict__ ptrs, void* lds) {
+__global__ __launch_bounds__(kTransposeThreads) void mmr_transpose_kernel(const mmr_transpose_chunk* __restrict__ chunks,
+                                                                          uint32_t n, void* const* __restrict__ ptrs,
+                                                                          uint32_t xcd_group) {
+  // 64 x 65 eight-byte elements is the largest tile (33,280 bytes); sixteen-byte
+  // elements use 32 x 33 tiles (16,896 bytes).
+  __shared__ alignas(16) uint64_t lds[64 * 65];
+  const uint32_t ci = chunk_index(blockIdx.x, xcd_group);
+  if (ci >= n) return;  // uniform over the workgroup: no barrier is skipped by part of it
   const mmr_transpose_chunk c = chunks[ci];
   gcchar* src = slot_base(ptrs, c.src_slot, c.src_off);
   gchar* dst = slot_base(ptrs, c.dst_slot, c.dst_off);
@@ -137,52 +131,41 @@ __device__ __forceinline__ void run_transpose(const mmr_transpose_chunk* __restr
   }
 }
 
-// One launch per plan: the grid is the four chunk tables back to back (each
-// padded to its XCD grouping); a workgroup finds its table by its block index
-// (wave-uniform branches) and runs one chunk of it.
-__global__ __launch_bounds__(kThreads) void mmr_reshard_kernel(PlanTables t, void* const* __restrict__ ptrs) {
-  // LDS is only allocated (at launch) when the plan has transpose chunks:
-  // 64 x 65 eight-byte elements is the largest tile (33,280 bytes).
-  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-  uint32_t b = blockIdx.x;
-  if (b < t.copy16.grid) {
-    const uint32_t ci = chunk_index(b, t.copy16.group);
-    if (ci < t.copy16.n) run_copy16(static_cast<const mmr_copy_chunk*>(t.copy16.chunks), ci, ptrs);
-    return;
-  }
-  b -= t.copy16.grid;
-  if (b < t.span.grid) {
-    const uint32_t ci = chunk_index(b, t.span.group);
-    if (ci < t.span.n) run_span(static_cast<const mmr_span_chunk*>(t.span.chunks), ci, ptrs);
-    return;
-  }
-  b -= t.span.grid;
-  if (b < t.generic.grid) {
-    const uint32_t ci = chunk_index(b, t.generic.group);
-    if (ci < t.generic.n) run_generic(static_cast<const mmr_copy_chunk*>(t.generic.chunks), ci, ptrs);
-    return;
-  }
-  b -= t.generic.grid;
-  const uint32_t ci = chunk_index(b, t.transpose.group);
-  if (ci < t.transpose.n)  // uniform over the workgroup: no barrier is skipped by part of it
-    run_transpose(static_cast<const mmr_transpose_chunk*>(t.transpose.chunks), ci, ptrs, lds);
-}
+hipError_t check_grid(int64_t n) { return (n < 0 || n > 0x7ff00000LL) ? hipErrorInvalidValue : hipSuccess; }
 
 }  // namespace
 
-void set_table(PlanTables::Table* t, const void* d_chunks, int64_t n, uint32_t xcd_mode) {
-  t->chunks = d_chunks;
-  t->n = static_cast<uint32_t>(n);
-  t->group = xcd_group_of(n, xcd_mode);
-  t->grid = n == 0 ? 0u : grid_size(n, t->group);
+// Launch shapes are the measured optimum on MI355X for 8 KiB (aligned) and
+// 4 KiB (generic) chunks: 256 threads, up to 8 (aligned) or 2 (generic) 16-byte
+// accesses in flight per lane before the first store.
+hipError_t launch_copy16(const mmr_copy_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
+                         hipStream_t stream) {
+  if (n == 0) return hipSuccess;
+  if (hipError_t e = check_grid(n)) return e;
+  const uint32_t group = xcd_group_of(n, xcd_mode);
+  hipLaunchKernelGGL((mmr_copy16_kernel<256, 8>), dim3(grid_size(n, group)), dim3(256), 0, stream, d_chunks,
+                     static_cast<uint32_t>(n), d_ptrs, group);
+  return hipGetLastError();
 }
 
-hipError_t launch_plan(const PlanTables& t, void* const* d_ptrs, hipStream_t stream) {
-  const uint64_t grid = static_cast<uint64_t>(t.copy16.grid) + t.span.grid + t.generic.grid + t.transpose.grid;
-  if (grid == 0) return hipSuccess;
-  if (grid > 0x7ff00000ULL) return hipErrorInvalidValue;
-  const size_t lds = t.transpose.n ? 64 * 65 * 8 : 0;
-  hipLaunchKernelGGL(mmr_reshard_kernel, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), lds, stream, t, d_ptrs);
+hipError_t launch_copy_generic(const mmr_copy_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
+                               hipStream_t stream) {
+  if (n == 0) return hipSuccess;
+  if (hipError_t e = check_grid(n)) return e;
+  const uint32_t group = xcd_group_of(n, xcd_mode);
+  // cacheable loads (a source line shared by two chunks is fetched once), nontemporal stores
+  hipLaunchKernelGGL((mmr_copy_generic_kernel<256, 2, false, true>), dim3(grid_size(n, group)), dim3(256), 0, stream,
+                     d_chunks, static_cast<uint32_t>(n), d_ptrs, group);
+  return hipGetLastError();
+}
+
+hipError_t launch_transpose(const mmr_transpose_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
+                            hipStream_t stream) {
+  if (n == 0) return hipSuccess;
+  if (hipError_t e = check_grid(n)) return e;
+  const uint32_t group = xcd_group_of(n, xcd_mode);
+  hipLaunchKernelGGL(mmr_transpose_kernel, dim3(grid_size(n, group)), dim3(kTransposeThreads), 0, stream, d_chunks,
+                     static_cast<uint32_t>(n), d_ptrs, group);
   return hipGetLastError();
 }
 

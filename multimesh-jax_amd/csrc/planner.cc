@@ -31,26 +31,8 @@ class Builder {
   Builder(mmr_plan* plan, uint32_t chunk_bytes, bool force_generic)
       : plan_(plan), chunk_bytes_(chunk_bytes), force_generic_(force_generic) {}
 
-  int64_t generic_chunk_bytes() const { return std::max<int64_t>(chunk_bytes_ / 2, 256); }
-
-  // statistics of one source-tile x destination-tile overlap
-  void count_box(const BoxDim* in, int rank, int itemsize) {
-    int64_t volume = 1;
-    for (int i = 0; i < rank; ++i) volume *= std::max<int64_t>(in[i].n, 0);
-    plan_->stats.n_boxes += 1;
-    plan_->stats.bytes_moved += volume * itemsize;
-  }
-
-  void add_span(const mmr_span_chunk& c, int itemsize) {
-    (void)itemsize;
-    for (uint32_t j = 0; j < c.n_pieces; ++j)
-      if (c.pieces[j].src_slot == MMR_SLOT_FILL) plan_->stats.bytes_filled += static_cast<int64_t>(c.pieces[j].w) * c.n_rows;
-    plan_->spans.push_back(c);
-  }
-
-  // count_box: false when the caller has already counted the overlap this box is (part of)
   void add_box(uint32_t src_slot, uint32_t dst_slot, int64_t src_off, int64_t dst_off, const BoxDim* in, int rank,
-               int itemsize, bool count = true) {
+               int itemsize) {
     std::vector<BoxDim> dims;
     int64_t volume = 1;
     for (int i = 0; i < rank; ++i) {
@@ -61,7 +43,7 @@ class Builder {
     const bool fill = src_slot == MMR_SLOT_FILL;
     if (fill) {
       plan_->stats.bytes_filled += volume * itemsize;
-    } else if (count) {
+    } else {
       plan_->stats.bytes_moved += volume * itemsize;
       plan_->stats.n_boxes += 1;
     }
@@ -107,7 +89,6 @@ class Builder {
     return best;
   }
 
- public:
   // Calls fn(src_delta, dst_delta) for every index combination of `dims`.
   template <class Fn>
   static void for_each_index(const std::vector<BoxDim>& dims, Fn&& fn) {
@@ -129,7 +110,6 @@ class Builder {
     }
   }
 
- private:
   void emit_copy(uint32_t src_slot, uint32_t dst_slot, int64_t so, int64_t dof, int64_t w, int64_t n1, int64_t n2,
                  int64_t s1, int64_t d1, int64_t s2, int64_t d2, bool fill) {
     mmr_copy_chunk c{};
@@ -159,7 +139,7 @@ class Builder {
     uint64_t bits = static_cast<uint64_t>(so | dof | w);
     for (const BoxDim& d : outer) bits |= static_cast<uint64_t>(d.s | d.d);
     const bool aligned = (bits & 15u) == 0 && !force_generic_;
-    const int64_t cb = aligned ? chunk_bytes_ : generic_chunk_bytes();
+    const int64_t cb = aligned ? chunk_bytes_ : std::max<int64_t>(chunk_bytes_ / 2, 256);
     if (w > cb) {
       // long rows: split columns into near-equal segments on 256-byte boundaries of the row
       const int64_t nseg = ceil_div(w, cb);
@@ -176,12 +156,35 @@ class Builder {
       emit_copy(src_slot, dst_slot, so, dof, w, 1, 1, 0, 0, 0, 0, fill);
       return;
     }
-    const BoxDim dim1 = outer[i1];
-    const int64_t n1 = std::min(dim1.n, rows);
+    BoxDim dim1 = outer[i1];
+    int64_t n1 = std::min(dim1.n, rows);
     BoxDim dim2{1, 0, 0};
     int64_t n2 = 1;
     int i2 = -1;
-    if (aligned && n1 == dim1.n && rows / n1 >= 2) {  // the generic kernel walks a single row dimension
+    // Rows that continue the run on the destination side along one dim (A) and on
+    // the source side along another (B), as a fused layout permutation produces:
+    // take a 2-D block so both sides see runs of several rows instead of one side
+    // seeing single rows at a large stride.
+    int ia = -1, ib = -1;
+    if (aligned && !fill && outer.size() >= 2) {
+      for (int i = 0; i < static_cast<int>(outer.size()); ++i) {
+        if (outer[i].d == w && outer[i].s != w) ia = i;
+        if (outer[i].s == w && outer[i].d != w) ib = i;
+      }
+    }
+    if (ia >= 0 && ib >= 0 && rows >= 4) {
+      const BoxDim da = outer[ia], db = outer[ib];
+      int64_t na = 1;
+      while (na * 2 <= da.n && na * na * 4 <= rows) na *= 2;  // about sqrt(rows), a power of two
+      if (da.n * da.n <= 4 * rows) na = da.n;                  // or the whole of a short dim
+      const int64_t nb = std::max<int64_t>(1, std::min(db.n, rows / na));
+      i1 = ia;
+      dim1 = da;
+      n1 = std::min(na, da.n);
+      i2 = ib;
+      dim2 = db;
+      n2 = nb;
+    } else if (aligned && n1 == dim1.n && rows / n1 >= 2) {  // the generic kernel walks a single row dimension
       i2 = pick_row_dim(outer, i1);
       if (i2 >= 0) {
         dim2 = outer[i2];
@@ -246,203 +249,59 @@ class Builder {
   bool force_generic_;
 };
 
-// One source-tile x destination-tile overlap of the tile being planned.
-struct TileBox {
-  uint32_t src_slot;
-  int64_t soff, doff;       // bytes: first element of the box in either buffer
-  BoxDim dims[kMaxRank];    // logical dim order
-  int64_t b_lo[kMaxRank];   // global index where the box starts
-};
-
-struct TileGeometry {
-  int64_t lo[kMaxRank], hi[kMaxRank], valid[kMaxRank];
-  int64_t t_lo[kMaxRank], t_n[kMaxRank];  // overlapping source tiles per dim
-  int64_t cstride[kMaxRank];              // box index = sum (t - t_lo) * cstride
-};
-
-// Zero the pad of a short tile: one slab per padded dim, dims taken in `order`:
-// the slab of a dim spans the valid extent of the dims before it and the whole
-// (padded) extent of the dims after it.  `skip_last`: the last dim's pad is
-// filled by other means (span chunks carry it as a piece without a source).
-void fill_pad(Builder& b, const Side& D, const TileGeometry& g, uint32_t dslot, const int* order, bool skip_last) {
-  const int rank = D.rank, item = D.itemsize;
-  for (int oi = 0; oi < rank - (skip_last ? 1 : 0); ++oi) {
-    const int i = order[oi];
-    if (g.valid[i] == D.ext[i]) continue;
-    BoxDim dims[kMaxRank];
-    for (int oj = 0; oj < rank; ++oj) {
-      const int j = order[oj];
-      const int64_t n = oj < oi ? g.valid[j] : (oj == oi ? D.ext[i] - g.valid[i] : D.ext[j]);
-      dims[j] = BoxDim{n, D.stride[j] * item, D.stride[j] * item};
-    }
-    b.add_box(MMR_SLOT_FILL, dslot, 0, g.valid[i] * D.stride[i] * item, dims, rank, item);
-  }
-}
-
-// Ragged rows (some offset, stride or width not a multiple of 16 bytes): plan the
-// tile as dense destination rows gathered from the source tiles that meet
-// inside a row, so every destination line is written whole by one workgroup.
-// Returns false when the tile does not fit the pattern; the caller then plans
-// it box by box.
-bool plan_tile_as_spans(Builder& b, const Side& S, const Side& D, const TileGeometry& g, uint32_t dslot,
-                        const std::vector<TileBox>& boxes) {
-  const int rank = S.rank, item = S.itemsize;
-  if (rank == 0 || boxes.empty()) return false;
-  int m = -1;
-  for (int i = 0; i < rank; ++i)
-    if (D.stride[i] == 1 && D.ext[i] > 1) m = i;
-  if (m < 0 || S.stride[m] != 1) return false;
-  // all aligned -> the aligned copy kernel is the better tool
-  uint64_t bits = 0;
-  for (const TileBox& bx : boxes) {
-    bits |= static_cast<uint64_t>(bx.soff | bx.doff);
-    for (int i = 0; i < rank; ++i) {
-      if (i == m) bits |= static_cast<uint64_t>(bx.dims[i].n * item);
-      else if (bx.dims[i].n > 1) bits |= static_cast<uint64_t>(bx.dims[i].s | bx.dims[i].d);
-    }
-  }
-  if ((bits & 15u) == 0) return false;
-  const bool pad_m = g.valid[m] < D.ext[m];
-  const int64_t n_pieces = g.t_n[m] + (pad_m ? 1 : 0);
-  if (n_pieces > MMR_SPAN_MAX_PIECES) return false;
-  const int64_t row_bytes = D.ext[m] * item;
-  const int64_t budget = b.generic_chunk_bytes();
-  if (row_bytes > 4 * budget) return false;  // very wide rows: split columns instead
-  int r = -1;  // the dim whose consecutive indices are consecutive destination rows
-  for (int i = 0; i < rank; ++i)
-    if (i != m && D.stride[i] == D.ext[m] && D.ext[i] > 1) r = i;
-  const int64_t rows_per_chunk = std::max<int64_t>(1, budget / row_bytes);
-
-  // pad of the other dims as whole-row slabs; the minor dim's pad rides in the spans
-  int order[kMaxRank], k = 0;
-  for (int i = 0; i < rank; ++i)
-    if (i != m) order[k++] = i;
-  order[k] = m;
-  fill_pad(b, D, g, dslot, order, /*skip_last=*/true);
-
-  // every combination of source tiles over the outer dims, every index of the outer dims but r
-  int64_t outer_combos = 1;
-  for (int i = 0; i < rank; ++i)
-    if (i != m) outer_combos *= g.t_n[i];
-  for (int64_t oc = 0; oc < outer_combos; ++oc) {
-    int64_t rem = oc, first = 0;  // index of the piece-0 box of this outer combination
-    for (int i = rank - 1; i >= 0; --i) {
-      if (i == m) continue;
-      first += (rem % g.t_n[i]) * g.cstride[i];
-      rem /= g.t_n[i];
-    }
-    const TileBox& b0 = boxes[static_cast<size_t>(first)];
-    std::vector<BoxDim> others;  // outer dims except r: every index is its own set of rows
-    std::vector<int> other_dim;
-    for (int i = 0; i < rank; ++i)
-      if (i != m && i != r) {
-        others.push_back(b0.dims[i]);
-        other_dim.push_back(i);
-      }
-    const int64_t n_r = r >= 0 ? b0.dims[r].n : 1;
-    const int64_t s_r = r >= 0 ? b0.dims[r].s : 0;
-    const int64_t d_r = r >= 0 ? b0.dims[r].d : 0;
-    Builder::for_each_index(others, [&](int64_t ds, int64_t dd) {
-      for (int64_t r0 = 0; r0 < n_r; r0 += rows_per_chunk) {
-        const int64_t n = std::min(rows_per_chunk, n_r - r0);
-        mmr_span_chunk c{};
-        c.dst_slot = dslot;
-        c.dst_off = static_cast<uint64_t>(b0.doff + dd + r0 * d_r);
-        c.row_bytes = static_cast<uint32_t>(row_bytes);
-        c.n_rows = static_cast<uint32_t>(n);
-        bool safe = true;
-        int64_t total = 0;
-        for (int64_t pj = 0; pj < g.t_n[m]; ++pj) {
-          const TileBox& bx = boxes[static_cast<size_t>(first + pj * g.cstride[m])];
-          mmr_span_piece& pc = c.pieces[c.n_pieces++];
-          pc.src_slot = bx.src_slot;
-          pc.w = static_cast<uint32_t>(bx.dims[m].n * item);
-          pc.src_off = static_cast<uint64_t>(bx.soff + ds + r0 * s_r);
-          pc.s1 = n > 1 ? s_r : 0;
-          total += pc.w;
-          // the kernel reads up to 15 bytes before and after every source run
-          if (pc.src_off < 15 || static_cast<int64_t>(pc.src_off) + (n - 1) * s_r + pc.w + 15 > S.shard_bytes) safe = false;
-        }
-        if (pad_m) {
-          mmr_span_piece& pc = c.pieces[c.n_pieces++];
-          pc.src_slot = MMR_SLOT_FILL;
-          pc.w = static_cast<uint32_t>((D.ext[m] - g.valid[m]) * item);
-          total += pc.w;
-        }
-        if (total != row_bytes) safe = false;  // cannot happen; keeps a malformed chunk off the GPU
-        if (safe) {
-          b.add_span(c, item);
-        } else {
-          // rows at the very start or end of a source buffer: move them piece by piece
-          for (uint32_t pj = 0; pj < c.n_pieces; ++pj) {
-            const mmr_span_piece& pc = c.pieces[pj];
-            int64_t col = 0;
-            for (uint32_t q = 0; q < pj; ++q) col += c.pieces[q].w;
-            BoxDim dims[2] = {BoxDim{n, pc.src_slot == MMR_SLOT_FILL ? row_bytes : s_r, row_bytes},
-                              BoxDim{pc.w / item, item, item}};
-            b.add_box(pc.src_slot, dslot, static_cast<int64_t>(pc.src_off), static_cast<int64_t>(c.dst_off) + col, dims, 2,
-                      item, /*count_box=*/false);
-          }
-        }
-      }
-    });
-  }
-  return true;
-}
-
-int plan_one_array(Builder& b, const Side& S, const Side& D, uint32_t slot_base, bool allow_spans) {
+int plan_one_array(Builder& b, const Side& S, const Side& D, uint32_t slot_base) {
   const int rank = S.rank;
   const int item = S.itemsize;
   for (int i = 0; i < rank; ++i)
     if (S.size[i] == 0) return MMR_OK;  // empty array: nothing to move, nothing to pad
-  int natural_order[kMaxRank];
-  for (int i = 0; i < rank; ++i) natural_order[i] = i;
   for (int64_t dd = 0; dd < D.dev_count; ++dd) {
     const uint32_t dslot = slot_base + static_cast<uint32_t>(S.dev_count + dd);
-    TileGeometry g;
+    int64_t lo[kMaxRank], hi[kMaxRank], valid[kMaxRank];
     bool padded = false, empty = false;
     for (int i = 0; i < rank; ++i) {
       const int64_t c = (dd / D.dev_stride[i]) % D.tiles[i];
-      g.lo[i] = std::min(c * D.ext[i], D.size[i]);
-      g.hi[i] = std::min(g.lo[i] + D.ext[i], D.size[i]);
-      g.valid[i] = g.hi[i] - g.lo[i];
-      padded |= g.valid[i] < D.ext[i];
-      empty |= g.valid[i] == 0;
+      lo[i] = std::min(c * D.ext[i], D.size[i]);
+      hi[i] = std::min(lo[i] + D.ext[i], D.size[i]);
+      valid[i] = hi[i] - lo[i];
+      padded |= valid[i] < D.ext[i];
+      empty |= valid[i] == 0;
     }
-    if (empty) {
-      if (padded) fill_pad(b, D, g, dslot, natural_order, false);
-      continue;
+    if (padded) {
+      // the pad of a short tile is rank slabs: dim i beyond its valid extent,
+      // dims before it inside theirs, dims after it whole
+      for (int i = 0; i < rank; ++i) {
+        if (valid[i] == D.ext[i]) continue;
+        BoxDim dims[kMaxRank];
+        for (int j = 0; j < rank; ++j) {
+          const int64_t n = j < i ? valid[j] : (j == i ? D.ext[i] - valid[i] : D.ext[j]);
+          dims[j] = BoxDim{n, D.stride[j] * item, D.stride[j] * item};
+        }
+        b.add_box(MMR_SLOT_FILL, dslot, 0, valid[i] * D.stride[i] * item, dims, rank, item);
+      }
     }
-    int64_t combos = 1;
-    for (int i = rank - 1; i >= 0; --i) {
-      g.t_lo[i] = g.lo[i] / S.ext[i];
-      g.t_n[i] = (g.hi[i] - 1) / S.ext[i] - g.t_lo[i] + 1;
-      g.cstride[i] = combos;
-      combos *= g.t_n[i];
+    if (empty) continue;
+    int64_t t_lo[kMaxRank], t_n[kMaxRank], combos = 1;
+    for (int i = 0; i < rank; ++i) {
+      t_lo[i] = lo[i] / S.ext[i];
+      t_n[i] = (hi[i] - 1) / S.ext[i] - t_lo[i] + 1;
+      combos *= t_n[i];
     }
-    std::vector<TileBox> boxes(static_cast<size_t>(combos));
     for (int64_t c = 0; c < combos; ++c) {
-      int64_t rem = c, sdev = 0;
-      TileBox& bx = boxes[static_cast<size_t>(c)];
-      bx.soff = bx.doff = 0;
+      int64_t rem = c, sdev = 0, soff = 0, doff = 0;
+      BoxDim dims[kMaxRank];
       for (int i = rank - 1; i >= 0; --i) {
-        const int64_t t = g.t_lo[i] + rem % g.t_n[i];
-        rem /= g.t_n[i];
+        const int64_t t = t_lo[i] + rem % t_n[i];
+        rem /= t_n[i];
         const int64_t s_lo = t * S.ext[i];
-        const int64_t b_lo = std::max(g.lo[i], s_lo);
-        const int64_t b_hi = std::min(g.hi[i], std::min(s_lo + S.ext[i], S.size[i]));
-        bx.dims[i] = BoxDim{b_hi - b_lo, S.stride[i] * item, D.stride[i] * item};
-        bx.b_lo[i] = b_lo;
-        bx.soff += (b_lo - s_lo) * S.stride[i] * item;
-        bx.doff += (b_lo - g.lo[i]) * D.stride[i] * item;
+        const int64_t b_lo = std::max(lo[i], s_lo);
+        const int64_t b_hi = std::min(hi[i], std::min(s_lo + S.ext[i], S.size[i]));
+        dims[i] = BoxDim{b_hi - b_lo, S.stride[i] * item, D.stride[i] * item};
+        soff += (b_lo - s_lo) * S.stride[i] * item;
+        doff += (b_lo - lo[i]) * D.stride[i] * item;
         sdev += t * S.dev_stride[i];  // of R source replicas the lowest device id is read
       }
-      bx.src_slot = slot_base + static_cast<uint32_t>(sdev);
-      b.count_box(bx.dims, rank, item);
+      b.add_box(slot_base + static_cast<uint32_t>(sdev), dslot, soff, doff, dims, rank, item);
     }
-    if (allow_spans && plan_tile_as_spans(b, S, D, g, dslot, boxes)) continue;
-    if (padded) fill_pad(b, D, g, dslot, natural_order, false);
-    for (const TileBox& bx : boxes) b.add_box(bx.src_slot, dslot, bx.soff, bx.doff, bx.dims, rank, item, false);
   }
   return MMR_OK;
 }
@@ -485,10 +344,23 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
     plan->srcs.push_back(srcs[a]);
     plan->dsts.push_back(dsts[a]);
     plan->slot_bases.push_back(plan->n_slots);
-    if (int rc = plan_one_array(builder, S, D, static_cast<uint32_t>(plan->n_slots),
-                                (options.flags & (MMR_PLAN_NO_SPANS | MMR_PLAN_ALL_GENERIC)) == 0))
-      return rc;
+    if (int rc = plan_one_array(builder, S, D, static_cast<uint32_t>(plan->n_slots))) return rc;
     plan->n_slots += S.dev_count + D.dev_count;
+  }
+  // A plan that is mostly ragged rows: its few aligned chunks ride along in the
+  // generic table (the generic kernel handles aligned rows too), one launch less.
+  if (!plan->generic.empty() && !plan->copy16.empty()) {
+    int64_t aligned_bytes = 0, generic_bytes = 0;
+    bool one_dim = true;
+    for (const mmr_copy_chunk& c : plan->copy16) {
+      aligned_bytes += static_cast<int64_t>(c.w) * c.n1 * c.n2;
+      one_dim &= c.n2 == 1;
+    }
+    for (const mmr_copy_chunk& c : plan->generic) generic_bytes += static_cast<int64_t>(c.w) * c.n1 * c.n2;
+    if (one_dim && aligned_bytes * 4 < generic_bytes) {
+      plan->generic.insert(plan->generic.end(), plan->copy16.begin(), plan->copy16.end());
+      plan->copy16.clear();
+    }
   }
   const uint32_t order = options.order ? options.order : 2;
   if (order == 2 || order == 3) {
@@ -498,11 +370,6 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
     auto cmp = [&](const mmr_copy_chunk& a, const mmr_copy_chunk& b) { return key(a) < key(b); };
     std::stable_sort(plan->copy16.begin(), plan->copy16.end(), cmp);
     std::stable_sort(plan->generic.begin(), plan->generic.end(), cmp);
-    std::stable_sort(plan->spans.begin(), plan->spans.end(), [order](const mmr_span_chunk& a, const mmr_span_chunk& b) {
-      return order == 2 ? std::make_pair(a.dst_slot, a.dst_off) < std::make_pair(b.dst_slot, b.dst_off)
-                        : std::make_pair(a.pieces[0].src_slot, a.pieces[0].src_off) <
-                              std::make_pair(b.pieces[0].src_slot, b.pieces[0].src_off);
-    });
     std::stable_sort(plan->transposes.begin(), plan->transposes.end(),
                      [order](const mmr_transpose_chunk& a, const mmr_transpose_chunk& b) {
                        return order == 2 ? std::make_pair(a.dst_slot, a.dst_off) < std::make_pair(b.dst_slot, b.dst_off)
@@ -513,12 +380,10 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
   plan->stats.n_copy16_chunks = static_cast<int64_t>(plan->copy16.size());
   plan->stats.n_copy_generic_chunks = static_cast<int64_t>(plan->generic.size());
   plan->stats.n_transpose_chunks = static_cast<int64_t>(plan->transposes.size());
-  plan->stats.n_span_chunks = static_cast<int64_t>(plan->spans.size());
   plan->stats.n_slots = plan->n_slots;
   plan->stats.table_bytes =
       static_cast<int64_t>((plan->copy16.size() + plan->generic.size()) * sizeof(mmr_copy_chunk) +
-                           plan->transposes.size() * sizeof(mmr_transpose_chunk) +
-                           plan->spans.size() * sizeof(mmr_span_chunk) + plan->n_slots * sizeof(void*));
+                           plan->transposes.size() * sizeof(mmr_transpose_chunk) + plan->n_slots * sizeof(void*));
   return MMR_OK;
 }
 
@@ -563,13 +428,6 @@ int64_t mmr_plan_get_transpose_chunks(const mmr_plan* plan, mmr_transpose_chunk*
   int64_t n = std::min<int64_t>(capacity, static_cast<int64_t>(plan->transposes.size()));
   if (out && n > 0) std::memcpy(out, plan->transposes.data(), sizeof(mmr_transpose_chunk) * n);
   return out ? n : static_cast<int64_t>(plan->transposes.size());
-}
-
-int64_t mmr_plan_get_span_chunks(const mmr_plan* plan, mmr_span_chunk* out, int64_t capacity) {
-  if (!plan) return 0;
-  int64_t n = std::min<int64_t>(capacity, static_cast<int64_t>(plan->spans.size()));
-  if (out && n > 0) std::memcpy(out, plan->spans.data(), sizeof(mmr_span_chunk) * n);
-  return out ? n : static_cast<int64_t>(plan->spans.size());
 }
 
 int64_t mmr_plan_get_slot_bases(const mmr_plan* plan, int64_t* out, int64_t capacity) {

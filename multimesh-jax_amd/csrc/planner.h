@@ -20,7 +20,6 @@ struct mmr_plan {
   std::vector<mmr_copy_chunk> copy16;   // every offset, stride and width a multiple of 16
   std::vector<mmr_copy_chunk> generic;  // anything else
   std::vector<mmr_transpose_chunk> transposes;
-  std::vector<mmr_span_chunk> spans;  // dense destination rows gathered from a few source pieces (ragged rows)
   mmr_plan_stats stats{};
 };
 

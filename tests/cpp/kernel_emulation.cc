@@ -195,35 +195,6 @@ int mmr_emulate_plan(const mmr_plan* plan, void* const* slot_ptrs, const size_t*
       }
     });
   }
-  if (g_error.empty()) {
-    const int64_t n = mmr_plan_get_span_chunks(plan, nullptr, 0);
-    std::vector<mmr_span_chunk> chunks(static_cast<size_t>(n));
-    mmr_plan_get_span_chunks(plan, chunks.data(), n);
-    for_each_chunk(n, xcd_mode == 0 ? 64 : xcd_mode, [&](uint32_t ci) {
-      const mmr_span_chunk& c = chunks[ci];
-      if (c.dst_slot >= n_slots || c.n_pieces < 1 || c.n_pieces > MMR_SPAN_MAX_PIECES) {
-        g_error = "malformed span chunk";
-        return;
-      }
-      uint8_t* dst = base(c.dst_slot, c.dst_off);
-      mmr::SpanSources<HostMem> srcs;
-      uint32_t total = 0;
-      for (uint32_t j = 0; j < MMR_SPAN_MAX_PIECES; ++j) {
-        const bool live = j < c.n_pieces && c.pieces[j].src_slot != MMR_SLOT_FILL;
-        if (live && c.pieces[j].src_slot >= n_slots) {
-          g_error = "span piece names a slot outside the pointer table";
-          return;
-        }
-        srcs.base[j] = live ? base(c.pieces[j].src_slot, c.pieces[j].src_off) : dst;
-        if (j < c.n_pieces) total += c.pieces[j].w;
-      }
-      if (total != c.row_bytes) {
-        g_error = "span pieces do not add up to the row";
-        return;
-      }
-      for (uint32_t tid = 0; tid < 256; ++tid) mmr::span_chunk<HostMem, 256>(c, srcs, dst, tid);
-    });
-  }
   if (bytes_loaded) *bytes_loaded = g_loaded;
   if (bytes_stored) *bytes_stored = g_stored;
   if (!g_error.empty()) {

@@ -48,23 +48,6 @@ def apply_plan(plan: "mm.Plan", buffers: Sequence[np.ndarray]) -> None:
             a = int(c["align"])
             for v in ("dst_off", "w", "d1", "d2") + (() if fill else ("src_off", "s1", "s2")):
                 assert int(c[v]) % a == 0, (v, c)
-    for c in plan.span_chunks():
-        dst = buffers[c["dst_slot"]]
-        assert sum(p["w"] for p in c["pieces"]) == c["row_bytes"]
-        for row in range(c["n_rows"]):
-            col = 0
-            for p in c["pieces"]:
-                do = c["dst_off"] + row * c["row_bytes"] + col
-                assert do + p["w"] <= dst.size
-                if p["src_slot"] == 0xFFFFFFFF:
-                    dst[do:do + p["w"]] = 0
-                else:
-                    src = buffers[p["src_slot"]]
-                    so = p["src_off"] + row * p["s1"]
-                    # the kernel may read 15 bytes either side of a run: that must stay inside the buffer
-                    assert so >= 15 and so + p["w"] + 15 <= src.size, (so, p, src.size)
-                    dst[do:do + p["w"]] = src[so:so + p["w"]]
-                col += p["w"]
     for c in plan.transpose_chunks():
         src = buffers[int(c["src_slot"])]
         dst = buffers[int(c["dst_slot"])]
