@@ -116,7 +116,8 @@ def measure(ctx, mm, workloads, args, config, with_parity=True):
         "achieved": alg_bytes / (kernel_ms / args.steps * 1e-3) / 1e9,
         "launches": launches,
         "plan": plan,
-        "kernel": "mmr_copy_generic_kernel" if generic or config in (5, 6) else "mmr_copy16_kernel",
+        "kernel": ("mmr_transpose_kernel" if plan is not None and plan["n_transpose_chunks"] > 0 else
+                   "mmr_copy_generic_kernel" if generic or config in (5, 6) else "mmr_copy16_kernel"),
         "n_arrays": len(arrays),
         "sets": len(sets),
     }

@@ -155,15 +155,15 @@ typedef struct {
   int64_t s2, d2;
 } mmr_copy_chunk;
 
-/* One batch of <=64x64-element tiles moved through LDS when source and
- * destination disagree on the minor-most dim.  x is contiguous in the source,
- * y is contiguous in the destination. */
+/* One batch of tiles moved through LDS when source and destination disagree on
+ * the minor-most dim.  x is contiguous in the source, y is contiguous in the
+ * destination.  Tile edge: 64 elements (128 for 1-byte, 32 for 16-byte elements). */
 typedef struct {
   uint32_t src_slot;
   uint32_t dst_slot;
   uint64_t src_off;
   uint64_t dst_off;
-  uint32_t nx, ny;   /* tile extent in elements, each <= 64 */
+  uint32_t nx, ny;   /* tile extent in elements, each at most the tile edge */
   uint32_t nb;       /* tiles along the batch dimension */
   uint32_t itemsize; /* 1, 2, 4, 8 or 16 */
   int64_t src_ystride, dst_xstride; /* bytes */

@@ -231,30 +231,116 @@ MMR_HD void generic_chunk(const mmr_copy_chunk& c, typename M::cptr src, typenam
 }
 
 // ---------------------------------------------------------------------------
-// Tile transpose: x is contiguous in the source, y in the destination.  Rows of
-// the tile are read along x into tile[y][x] (row pitch TILE + 1 elements to
-// spread the column reads over the LDS banks) and written along y.  The caller
-// puts a workgroup barrier between the two phases and after the store phase.
+// Tile transpose: x is contiguous in the source, y in the destination.  The
+// caller puts a workgroup barrier between the load and the store phase and
+// after the store phase.  Tile edge in elements: 128 for 1-byte, 64 for 2/4/8-
+// byte, 32 for 16-byte elements.
+//
+// Vector path (tile 16-byte aligned on both sides, extents multiples of the
+// vector width): every global access is a 16-byte vector.  A lane loads one
+// vector of a source row, scatters its elements into LDS laid out [x][y] (row
+// pitch EDGE + elements-per-vector, so rows stay 16-byte aligned), and after the
+// barrier reads one 16-byte vector of an LDS row = consecutive y of one x and
+// stores it to the destination row x.  All loads of a thread are issued before
+// its first LDS write.
+//
+// Element path (anything else, e.g. ragged edge tiles): one element per lane,
+// LDS laid out [y][x] with pitch EDGE + 1.
 // ---------------------------------------------------------------------------
-template <class M, typename T, int TILE, int THREADS>
-MMR_HD void transpose_load(const mmr_transpose_chunk& c, typename M::cptr src, uint32_t b, T (*tile)[TILE + 1],
-                           uint32_t tid) {
+template <int ITEM>
+struct TransposeTile {
+  static constexpr int kEdge = ITEM == 1 ? 128 : (ITEM == 16 ? 32 : 64);
+  static constexpr int kVec = 16 / ITEM;           // elements per 16-byte vector
+  static constexpr int kPitch = kEdge + kVec;      // vector path, elements
+  static constexpr int kPitch1 = kEdge + 1;        // element path, elements
+  static constexpr int kLdsBytes = kEdge * kPitch * ITEM;
+};
+constexpr int kTransposeLdsBytes = 64 * 66 * 8;  // the largest of TransposeTile<>::kLdsBytes (8-byte elements)
+
+MMR_HD bool transpose_is_vector(const mmr_transpose_chunk& c) {
+  const uint32_t vec = 16u / c.itemsize;
+  const uint64_t bits = c.src_off | c.dst_off | static_cast<uint64_t>(c.src_ystride) | static_cast<uint64_t>(c.dst_xstride) |
+                        static_cast<uint64_t>(c.src_bstride) | static_cast<uint64_t>(c.dst_bstride);
+  return (bits & 15u) == 0 && c.nx % vec == 0 && c.ny % vec == 0;
+}
+
+template <typename T>
+MMR_HD T element_of(const V16& v, int i) {
+  // i is a compile-time constant after unrolling
+  if constexpr (sizeof(T) == 16) {
+    return v;
+  } else if constexpr (sizeof(T) == 8) {
+    return i == 0 ? (static_cast<uint64_t>(v.x) | (static_cast<uint64_t>(v.y) << 32))
+                  : (static_cast<uint64_t>(v.z) | (static_cast<uint64_t>(v.w) << 32));
+  } else {
+    constexpr int per = 4 / static_cast<int>(sizeof(T));  // elements per dword
+    const uint32_t d = i / per == 0 ? v.x : (i / per == 1 ? v.y : (i / per == 2 ? v.z : v.w));
+    return static_cast<T>(d >> (8 * static_cast<int>(sizeof(T)) * (i % per)));
+  }
+}
+
+template <class M, typename T, int THREADS>
+MMR_HD void transpose_load_vec(const mmr_transpose_chunk& c, typename M::cptr src, uint32_t b, T* lds, uint32_t tid) {
+  typedef TransposeTile<sizeof(T)> G;
+  constexpr int kRowVecs = G::kEdge / G::kVec;                // vectors per full source row of the tile
+  constexpr int kPerThread = G::kEdge * kRowVecs / THREADS;   // vectors per thread
+  typename M::cptr s = src + b * c.src_bstride;
+  V16 v[kPerThread];
+#pragma unroll
+  for (int k = 0; k < kPerThread; ++k) {
+    const uint32_t vi = tid + k * THREADS;
+    const uint32_t y = vi / kRowVecs, xv = vi % kRowVecs;
+    if (y < c.ny && xv * G::kVec < c.nx) v[k] = M::load16(s + (y * c.src_ystride + static_cast<int64_t>(xv) * 16));
+  }
+#pragma unroll
+  for (int k = 0; k < kPerThread; ++k) {
+    const uint32_t vi = tid + k * THREADS;
+    const uint32_t y = vi / kRowVecs, xv = vi % kRowVecs;
+    if (y < c.ny && xv * G::kVec < c.nx) {
+#pragma unroll
+      for (int i = 0; i < G::kVec; ++i) lds[(xv * G::kVec + i) * G::kPitch + y] = element_of<T>(v[k], i);
+    }
+  }
+}
+
+template <class M, typename T, int THREADS>
+MMR_HD void transpose_store_vec(const mmr_transpose_chunk& c, typename M::ptr dst, uint32_t b, const T* lds, uint32_t tid) {
+  typedef TransposeTile<sizeof(T)> G;
+  constexpr int kRowVecs = G::kEdge / G::kVec;  // vectors per full destination row of the tile
+  constexpr int kPerThread = G::kEdge * kRowVecs / THREADS;
+  typename M::ptr d = dst + b * c.dst_bstride;
+#pragma unroll
+  for (int k = 0; k < kPerThread; ++k) {
+    const uint32_t vi = tid + k * THREADS;
+    const uint32_t x = vi / kRowVecs, yv = vi % kRowVecs;
+    if (x < c.nx && yv * G::kVec < c.ny) {
+      const V16 v = *reinterpret_cast<const V16*>(&lds[x * G::kPitch + yv * G::kVec]);  // 16-byte aligned by construction
+      M::store16(d + (x * c.dst_xstride + static_cast<int64_t>(yv) * 16), v);
+    }
+  }
+}
+
+template <class M, typename T, int THREADS>
+MMR_HD void transpose_load(const mmr_transpose_chunk& c, typename M::cptr src, uint32_t b, T* lds, uint32_t tid) {
+  typedef TransposeTile<sizeof(T)> G;
   typename M::cptr s = src + b * c.src_bstride;
   const uint32_t n = c.nx * c.ny;
   for (uint32_t i = tid; i < n; i += THREADS) {
     const uint32_t y = i / c.nx, x = i - y * c.nx;
-    tile[y][x] = M::template loadu<T>(s + (y * c.src_ystride + static_cast<int64_t>(x) * static_cast<int64_t>(sizeof(T))));
+    lds[y * G::kPitch1 + x] =
+        M::template loadu<T>(s + (y * c.src_ystride + static_cast<int64_t>(x) * static_cast<int64_t>(sizeof(T))));
   }
 }
 
-template <class M, typename T, int TILE, int THREADS>
-MMR_HD void transpose_store(const mmr_transpose_chunk& c, typename M::ptr dst, uint32_t b, T (*tile)[TILE + 1],
-                            uint32_t tid) {
+template <class M, typename T, int THREADS>
+MMR_HD void transpose_store(const mmr_transpose_chunk& c, typename M::ptr dst, uint32_t b, const T* lds, uint32_t tid) {
+  typedef TransposeTile<sizeof(T)> G;
   typename M::ptr d = dst + b * c.dst_bstride;
   const uint32_t n = c.nx * c.ny;
   for (uint32_t i = tid; i < n; i += THREADS) {
     const uint32_t x = i / c.ny, y = i - x * c.ny;
-    M::template storeu<T>(d + (x * c.dst_xstride + static_cast<int64_t>(y) * static_cast<int64_t>(sizeof(T))), tile[y][x]);
+    M::template storeu<T>(d + (x * c.dst_xstride + static_cast<int64_t>(y) * static_cast<int64_t>(sizeof(T))),
+                          lds[y * G::kPitch1 + x]);
   }
 }
 

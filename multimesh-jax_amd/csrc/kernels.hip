@@ -99,14 +99,17 @@ __global__ __launch_bounds__(THREADS) void mmr_copy_generic_kernel(const mmr_cop
 
 constexpr int kTransposeThreads = 256;
 
-template <typename T, int TILE>
+template <typename T>
 __device__ __forceinline__ void transpose_tiles(const mmr_transpose_chunk& c, gcchar* src, gchar* dst, void* lds_raw) {
   typedef DeviceMem<true, true> M;
-  T(*tile)[TILE + 1] = reinterpret_cast<T(*)[TILE + 1]>(lds_raw);
+  T* lds = static_cast<T*>(lds_raw);
+  const bool vec = transpose_is_vector(c);  // wave-uniform
   for (uint32_t b = 0; b < c.nb; ++b) {
-    transpose_load<M, T, TILE, kTransposeThreads>(c, src, b, tile, threadIdx.x);
+    if (vec) transpose_load_vec<M, T, kTransposeThreads>(c, src, b, lds, threadIdx.x);
+    else transpose_load<M, T, kTransposeThreads>(c, src, b, lds, threadIdx.x);
     __syncthreads();
-    transpose_store<M, T, TILE, kTransposeThreads>(c, dst, b, tile, threadIdx.x);
+    if (vec) transpose_store_vec<M, T, kTransposeThreads>(c, dst, b, lds, threadIdx.x);
+    else transpose_store<M, T, kTransposeThreads>(c, dst, b, lds, threadIdx.x);
     __syncthreads();
   }
 }
@@ -114,20 +117,18 @@ __device__ __forceinline__ void transpose_tiles(const mmr_transpose_chunk& c, gc
 __global__ __launch_bounds__(kTransposeThreads) void mmr_transpose_kernel(const mmr_transpose_chunk* __restrict__ chunks,
                                                                           uint32_t n, void* const* __restrict__ ptrs,
                                                                           uint32_t xcd_group) {
-  // 64 x 65 eight-byte elements is the largest tile (33,280 bytes); sixteen-byte
-  // elements use 32 x 33 tiles (16,896 bytes).
-  __shared__ alignas(16) uint64_t lds[64 * 65];
+  __shared__ alignas(16) uint8_t lds[kTransposeLdsBytes];
   const uint32_t ci = chunk_index(blockIdx.x, xcd_group);
   if (ci >= n) return;  // uniform over the workgroup: no barrier is skipped by part of it
   const mmr_transpose_chunk c = chunks[ci];
   gcchar* src = slot_base(ptrs, c.src_slot, c.src_off);
   gchar* dst = slot_base(ptrs, c.dst_slot, c.dst_off);
   switch (c.itemsize) {  // wave-uniform
-    case 1: transpose_tiles<uint8_t, 64>(c, src, dst, lds); break;
-    case 2: transpose_tiles<uint16_t, 64>(c, src, dst, lds); break;
-    case 4: transpose_tiles<uint32_t, 64>(c, src, dst, lds); break;
-    case 8: transpose_tiles<uint64_t, 64>(c, src, dst, lds); break;
-    default: transpose_tiles<V16, 32>(c, src, dst, lds); break;
+    case 1: transpose_tiles<uint8_t>(c, src, dst, lds); break;
+    case 2: transpose_tiles<uint16_t>(c, src, dst, lds); break;
+    case 4: transpose_tiles<uint32_t>(c, src, dst, lds); break;
+    case 8: transpose_tiles<uint64_t>(c, src, dst, lds); break;
+    default: transpose_tiles<V16>(c, src, dst, lds); break;
   }
 }
 

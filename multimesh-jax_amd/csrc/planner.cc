@@ -208,7 +208,7 @@ class Builder {
 
   void lower_transpose(uint32_t src_slot, uint32_t dst_slot, int64_t so, int64_t dof, const std::vector<BoxDim>& dims,
                        int x, int y, int itemsize) {
-    const int64_t tile = itemsize == 16 ? kTransposeTile / 2 : kTransposeTile;
+    const int64_t tile = itemsize == 1 ? 2 * kTransposeTile : (itemsize == 16 ? kTransposeTile / 2 : kTransposeTile);
     const BoxDim dx = dims[x], dy = dims[y];
     std::vector<BoxDim> outer;
     for (int i = 0; i < static_cast<int>(dims.size()); ++i)

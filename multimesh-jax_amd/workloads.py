@@ -14,7 +14,7 @@ from typing import Dict, List, Optional, Sequence
 
 import numpy as np
 
-ITEMSIZE = {"F32": 4, "BF16": 2, "S32": 4, "F8E4M3FN": 1, "U8": 1, "U16": 2, "U32": 4}
+ITEMSIZE = {"F32": 4, "BF16": 2, "S32": 4, "F8E4M3FN": 1, "U8": 1, "U16": 2, "U32": 4, "F64": 8, "C128": 16}
 
 
 def _side(shape: Sequence[int], sharding: Sequence[int], dev_start: int, replication: int = 1,
@@ -104,6 +104,11 @@ def config(index: int, scale: int = 1) -> List[dict]:
     if index == 12:  # probe: ragged destination rows of 4-byte elements from one source tile
         b = (44032 // s, 1025)
         return [_array("probe_s32_1to5", "S32", b, _side(b, (1, 1), 0), _side(b, (1, 5), 3), 6, "raw")]
+    if index in (13, 14, 15):  # transposed destination layout: rows 4-way, row-major -> columns 4-way, column-major
+        type_ = {13: "BF16", 14: "F32", 15: "U8"}[index]
+        shape = (8192 // s, 8192 // s)
+        return [_array("transposed", type_, shape, _side(shape, (4, 1), 0),
+                       _side(shape, (1, 4), 4, minor_to_major=(0, 1)), 13, "raw")]
     if index == 7:  # probe: 4-byte elements, uneven 3-way -> 5-way (dword-aligned, not 16-byte-aligned runs)
         b = (11008 // s, 1025)
         return [_array("probe_s32", "S32", b, _side(b, (1, 3), 0), _side(b, (1, 5), 3), 7, "raw")]

@@ -75,13 +75,24 @@ struct HostMem {
   static uintptr_t addr(ptr p) { return reinterpret_cast<uintptr_t>(p); }
 };
 
-template <typename T, int TILE>
+template <typename T>
 void run_transpose(const mmr_transpose_chunk& c, const uint8_t* src, uint8_t* dst) {
   constexpr int kThreads = 256;
-  static thread_local T tile[TILE][TILE + 1];
+  alignas(16) static thread_local uint8_t lds_raw[mmr::kTransposeLdsBytes];
+  static_assert(mmr::TransposeTile<sizeof(T)>::kLdsBytes <= mmr::kTransposeLdsBytes, "LDS tile too large");
+  static_assert(mmr::TransposeTile<sizeof(T)>::kEdge * mmr::TransposeTile<sizeof(T)>::kPitch1 * sizeof(T) <=
+                    mmr::kTransposeLdsBytes, "LDS tile too large");
+  T* lds = reinterpret_cast<T*>(lds_raw);
+  const bool vec = mmr::transpose_is_vector(c);
   for (uint32_t b = 0; b < c.nb; ++b) {
-    for (uint32_t tid = 0; tid < kThreads; ++tid) mmr::transpose_load<HostMem, T, TILE, kThreads>(c, src, b, tile, tid);
-    for (uint32_t tid = 0; tid < kThreads; ++tid) mmr::transpose_store<HostMem, T, TILE, kThreads>(c, dst, b, tile, tid);
+    for (uint32_t tid = 0; tid < kThreads; ++tid) {
+      if (vec) mmr::transpose_load_vec<HostMem, T, kThreads>(c, src, b, lds, tid);
+      else mmr::transpose_load<HostMem, T, kThreads>(c, src, b, lds, tid);
+    }
+    for (uint32_t tid = 0; tid < kThreads; ++tid) {
+      if (vec) mmr::transpose_store_vec<HostMem, T, kThreads>(c, dst, b, lds, tid);
+      else mmr::transpose_store<HostMem, T, kThreads>(c, dst, b, lds, tid);
+    }
   }
 }
 
@@ -181,17 +192,17 @@ int mmr_emulate_plan(const mmr_plan* plan, void* const* slot_ptrs, const size_t*
       }
       const uint8_t* src = base(c.src_slot, c.src_off);
       uint8_t* dst = base(c.dst_slot, c.dst_off);
-      const uint32_t tile = c.itemsize == 16 ? 32 : 64;
+      const uint32_t tile = c.itemsize == 1 ? 128 : (c.itemsize == 16 ? 32 : 64);
       if (c.nx > tile || c.ny > tile) {
         g_error = "transpose tile larger than the LDS tile";
         return;
       }
       switch (c.itemsize) {
-        case 1: run_transpose<uint8_t, 64>(c, src, dst); break;
-        case 2: run_transpose<uint16_t, 64>(c, src, dst); break;
-        case 4: run_transpose<uint32_t, 64>(c, src, dst); break;
-        case 8: run_transpose<uint64_t, 64>(c, src, dst); break;
-        default: run_transpose<mmr::V16, 32>(c, src, dst); break;
+        case 1: run_transpose<uint8_t>(c, src, dst); break;
+        case 2: run_transpose<uint16_t>(c, src, dst); break;
+        case 4: run_transpose<uint32_t>(c, src, dst); break;
+        case 8: run_transpose<uint64_t>(c, src, dst); break;
+        default: run_transpose<mmr::V16>(c, src, dst); break;
       }
     });
   }

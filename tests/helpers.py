@@ -52,7 +52,8 @@ def apply_plan(plan: "mm.Plan", buffers: Sequence[np.ndarray]) -> None:
         src = buffers[int(c["src_slot"])]
         dst = buffers[int(c["dst_slot"])]
         it = int(c["itemsize"])
-        assert int(c["nx"]) <= 64 and int(c["ny"]) <= 64
+        edge = {1: 128, 16: 32}.get(it, 64)
+        assert int(c["nx"]) <= edge and int(c["ny"]) <= edge
         for b in range(int(c["nb"])):
             for y in range(int(c["ny"])):
                 for x in range(int(c["nx"])):

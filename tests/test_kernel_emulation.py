@@ -92,3 +92,26 @@ def test_ragged_rows_through_the_kernel_code(a, chunk_bytes, shape):
     if a["shape"][1] == 1 and (a["src"]["dims"][1][1] > 1 or a["dst"]["dims"][1][1] > 1):
         return  # trailing {1, R} would read as a replication entry
     _check([a], [g], chunk_bytes=chunk_bytes, shape=shape)
+
+
+@pytest.mark.parametrize("type_", ["U8", "BF16", "F32", "F64", "C128"])
+@pytest.mark.parametrize("shape", [(256, 384), (192, 200), (130, 256)])
+def test_transposed_layout_vector_and_element_tiles(type_, shape):
+    """Aligned tiles take the 16-byte vector path, ragged edge tiles the element path."""
+    from oracle import reshard_oracle as ro
+    item = ro.ITEMSIZE[type_]
+    a = {"name": "t", "type": type_, "shape": shape,
+         "src": {"dims": [(shape[0], 2, 0), (shape[1], 1, 1)], "dev_start": 0, "dev_count": 2},
+         "dst": {"dims": [(shape[0], 1, 0), (shape[1], 2, 1)], "dev_start": 2, "dev_count": 2, "minor_to_major": [0, 1]},
+         "seed": 0, "dist": "raw"}
+    rng = np.random.Generator(np.random.PCG64(31))
+    g = rng.integers(0, 256, size=int(np.prod(shape)) * item, dtype=np.uint8).view(ro.raw_dtype(type_)).reshape(shape)
+    plan = _check([a], [g])
+    assert plan.stats["n_transpose_chunks"] > 0
+
+
+def test_transposed_benchmark_workloads_scaled():
+    for index in (13, 14, 15):
+        arrays = workloads.config(index, 16)
+        gs = [workloads.generate(a) for a in arrays]
+        _check(arrays, gs)
