@@ -34,6 +34,7 @@ struct DevicePlan {
   mmr_copy_chunk* d_copy16 = nullptr;
   mmr_copy_chunk* d_generic = nullptr;
   mmr_transpose_chunk* d_transposes = nullptr;
+  uint32_t max_transpose_itemsize = 1;
 };
 
 struct Binding {
@@ -133,6 +134,8 @@ int get_plan(mmr_context* ctx, const std::vector<mmr_sharded_shape>& srcs, const
   if (int rc = upload(ctx, dp->plan.copy16, &dp->d_copy16)) return rc;
   if (int rc = upload(ctx, dp->plan.generic, &dp->d_generic)) return rc;
   if (int rc = upload(ctx, dp->plan.transposes, &dp->d_transposes)) return rc;
+  for (const mmr_transpose_chunk& c : dp->plan.transposes)
+    dp->max_transpose_itemsize = std::max(dp->max_transpose_itemsize, c.itemsize);
   ctx->stats.plans_built += 1;
   *out = dp.get();
   ctx->plans.emplace(std::move(key), std::move(dp));
@@ -202,7 +205,7 @@ int reshard_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* d
   MMR_HIP(mmr::launch_copy_generic(dp->d_generic, static_cast<int64_t>(p.generic.size()), binding->d_ptrs, xm == 0 ? 2 : xm,
                                    ctx->stream));
   MMR_HIP(mmr::launch_transpose(dp->d_transposes, static_cast<int64_t>(p.transposes.size()), binding->d_ptrs, xm,
-                                ctx->stream));
+                                dp->max_transpose_itemsize, ctx->stream));
   ctx->stats.kernel_launches += (p.copy16.empty() ? 0 : 1) + (p.generic.empty() ? 0 : 1) + (p.transposes.empty() ? 0 : 1);
   return MMR_OK;
 }

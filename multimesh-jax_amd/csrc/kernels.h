@@ -20,8 +20,9 @@ hipError_t launch_copy16(const mmr_copy_chunk* d_chunks, int64_t n, void* const*
 hipError_t launch_copy_generic(const mmr_copy_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
                                hipStream_t stream);
 // LDS-staged tile transposes.
+// max_itemsize: widest element among the chunks (sizes the LDS tile).
 hipError_t launch_transpose(const mmr_transpose_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
-                            hipStream_t stream);
+                            uint32_t max_itemsize, hipStream_t stream);
 
 }  // namespace mmr
 

@@ -12,6 +12,7 @@
 // emulation the tests run.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdint>
 
 #include "chunk_ops.h"
@@ -117,7 +118,9 @@ __device__ __forceinline__ void transpose_tiles(const mmr_transpose_chunk& c, gc
 __global__ __launch_bounds__(kTransposeThreads) void mmr_transpose_kernel(const mmr_transpose_chunk* __restrict__ chunks,
                                                                           uint32_t n, void* const* __restrict__ ptrs,
                                                                           uint32_t xcd_group) {
-  __shared__ alignas(16) uint8_t lds[kTransposeLdsBytes];
+  // sized at launch for the widest element in the table (5 KiB for 1-byte up to
+  // 33 KiB for 8-byte elements), so narrow types keep full occupancy
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const uint32_t ci = chunk_index(blockIdx.x, xcd_group);
   if (ci >= n) return;  // uniform over the workgroup: no barrier is skipped by part of it
   const mmr_transpose_chunk c = chunks[ci];
@@ -160,12 +163,25 @@ hipError_t launch_copy_generic(const mmr_copy_chunk* d_chunks, int64_t n, void* 
   return hipGetLastError();
 }
 
+size_t transpose_lds_bytes(uint32_t itemsize) {
+  switch (itemsize) {
+    case 1: return TransposeTile<1>::kLdsBytes;
+    case 2: return TransposeTile<2>::kLdsBytes;
+    case 4: return TransposeTile<4>::kLdsBytes;
+    case 8: return TransposeTile<8>::kLdsBytes;
+    default: return TransposeTile<16>::kLdsBytes;
+  }
+}
+
 hipError_t launch_transpose(const mmr_transpose_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
-                            hipStream_t stream) {
+                            uint32_t max_itemsize, hipStream_t stream) {
   if (n == 0) return hipSuccess;
   if (hipError_t e = check_grid(n)) return e;
   const uint32_t group = xcd_group_of(n, xcd_mode);
-  hipLaunchKernelGGL(mmr_transpose_kernel, dim3(grid_size(n, group)), dim3(kTransposeThreads), 0, stream, d_chunks,
+  // the element path's [y][x] tile (pitch edge + 1) is never larger than the vector path's for the same type
+  size_t lds = 0;
+  for (uint32_t item = 1; item <= 16 && item <= max_itemsize; item *= 2) lds = std::max(lds, transpose_lds_bytes(item));
+  hipLaunchKernelGGL(mmr_transpose_kernel, dim3(grid_size(n, group)), dim3(kTransposeThreads), lds, stream, d_chunks,
                      static_cast<uint32_t>(n), d_ptrs, group);
   return hipGetLastError();
 }
