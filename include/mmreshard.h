@@ -226,6 +226,23 @@ int mmr_context_set_plan_options(mmr_context* ctx, const mmr_plan_options* optio
  * the descriptor's device list (zero-filled). */
 int mmr_store_create(mmr_context* ctx, const mmr_sharded_shape* shape, const char* name, uint32_t flags,
                      mmr_store** out);
+/* Zero-copy import (what AssembleShards' "TODO: do the slicing" flat copy,
+ * zuku_execute_context_impl.cc:405-415, would become when the native PjRt
+ * shards may be used in place): a store whose buffer of device dev_start + k IS
+ * device_ptrs[k] (caller-owned, 16-byte aligned, at least mmr_shard_bytes
+ * long).  mmr_store_free on it waits for pending work and frees nothing. */
+int mmr_store_adopt(mmr_context* ctx, const mmr_sharded_shape* shape, const char* name, void* const* device_ptrs,
+                    mmr_store** out);
+
+/* OffloadDtoH / OffloadHtoD, zuku_execute_context.h:61-68,
+ * zuku_execute_context_impl.cc:162-211: move every buffer of the store to
+ * pinned host memory and release the device memory / bring it back.  Blocking.
+ * An offloaded store cannot be resharded, assembled or sliced (the mock's
+ * invariant, mm_mock_mm_xla.cc:347-356); mmr_store_read_shard still works. */
+int mmr_store_offload(mmr_context* ctx, mmr_store* store);
+int mmr_store_reload(mmr_context* ctx, mmr_store* store);
+int mmr_store_is_offloaded(const mmr_store* store, int32_t* out);
+
 /* Free, zuku_execute_context_impl.cc:504-515 (keep_in_cache: buffers go back to
  * the per-shape cache); Destroy, :356-361. The handle is dead afterwards. */
 int mmr_store_free(mmr_context* ctx, mmr_store* store, int32_t keep_in_cache);
@@ -267,6 +284,17 @@ int mmr_reshard(mmr_context* ctx, mmr_store* src, mmr_store* dst);
  * mm_pjrt_executable.cc:616-658). */
 int mmr_reshard_batch(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int32_t n);
 
+/* Build and upload the plan of n descriptor pairs (one batch) ahead of the first
+ * reshard, i.e. when the schedule entry is created (MpmdScheduler::AddReshardTask,
+ * mpmd_partition.cc:340-351) rather than when it first executes. */
+int mmr_context_prepare(mmr_context* ctx, const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int32_t n);
+
+/* Ordering against other streams without blocking the host, as the plugin ties
+ * XLA's stream to the runtime's (RecordCuEvent, cuda_utils.cu.cc:78-83): the
+ * context's stream waits for a caller's hipEvent_t / records one. */
+int mmr_context_wait_event(mmr_context* ctx, void* hip_event);
+int mmr_context_record_event(mmr_context* ctx, void* hip_event);
+
 /* Blocks until everything queued on the context's stream is done. */
 int mmr_sync(mmr_context* ctx);
 
@@ -286,6 +314,8 @@ typedef struct {
   int64_t bytes_high_watermark;
   int64_t stores_live;
   int64_t cache_hits;      /* store buffers served from the per-shape cache */
+  int64_t host_bytes_allocated; /* pinned host bytes of offloaded stores */
+  int64_t host_bytes_high_watermark;
 } mmr_context_stats;
 int mmr_context_get_stats(mmr_context* ctx, mmr_context_stats* out);
 /* Stats of the cached plan of a store pair (builds it if needed). */

@@ -89,7 +89,8 @@ class PlanStats(C.Structure):
 class ContextStats(C.Structure):
     _fields_ = [(n, C.c_int64) for n in (
         "plans_built", "plan_cache_hits", "bindings_built", "binding_cache_hits", "kernel_launches",
-        "reshard_calls", "bytes_allocated", "bytes_high_watermark", "stores_live", "cache_hits")]
+        "reshard_calls", "bytes_allocated", "bytes_high_watermark", "stores_live", "cache_hits",
+        "host_bytes_allocated", "host_bytes_high_watermark")]
 
     def as_dict(self):
         return {n: getattr(self, n) for n, _ in self._fields_}
@@ -127,6 +128,13 @@ PROTOTYPES = {
     "mmr_context_stream": (C.c_int, [VP, P(VP)]),
     "mmr_context_set_plan_options": (C.c_int, [VP, P(PlanOptions)]),
     "mmr_store_create": (C.c_int, [VP, P(ShardedShape), C.c_char_p, C.c_uint32, P(VP)]),
+    "mmr_store_adopt": (C.c_int, [VP, P(ShardedShape), C.c_char_p, P(VP), P(VP)]),
+    "mmr_store_offload": (C.c_int, [VP, VP]),
+    "mmr_store_reload": (C.c_int, [VP, VP]),
+    "mmr_store_is_offloaded": (C.c_int, [VP, P(I32)]),
+    "mmr_context_prepare": (C.c_int, [VP, P(ShardedShape), P(ShardedShape), I32]),
+    "mmr_context_wait_event": (C.c_int, [VP, VP]),
+    "mmr_context_record_event": (C.c_int, [VP, VP]),
     "mmr_store_free": (C.c_int, [VP, VP, I32]),
     "mmr_clear_store_cache": (C.c_int, [VP]),
     "mmr_store_assemble": (C.c_int, [VP, VP, I64, VP, C.c_size_t, I32]),

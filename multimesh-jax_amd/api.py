@@ -303,6 +303,34 @@ class ReshardContext:
             B.check(self._lib.mmr_store_assemble(self._h, store._h, device, C.c_void_p(int(data)), size, 1))
         return store
 
+    def AdoptShards(self, shape: B.ShardedShape, device_ptrs: Sequence[int], name: Optional[str] = None) -> StoreHandle:
+        """Zero-copy import: device_ptrs[k] becomes the buffer of device dev_start + k."""
+        h = C.c_void_p()
+        arr = (C.c_void_p * max(len(device_ptrs), 1))(*[C.c_void_p(int(p)) for p in device_ptrs])
+        if len(device_ptrs) != shape.dev_count:
+            raise ValueError("one pointer per device of the descriptor")
+        B.check(self._lib.mmr_store_adopt(self._h, C.byref(shape), name.encode() if name else None, arr, C.byref(h)))
+        return StoreHandle(self, h, shape, name or "anonymous")
+
+    def OffloadDtoH(self, to_offload: Sequence[StoreHandle]) -> None:
+        for s in to_offload:
+            B.check(self._lib.mmr_store_offload(self._h, s._h))
+
+    def OffloadHtoD(self, to_offload: Sequence[StoreHandle]) -> None:
+        for s in to_offload:
+            B.check(self._lib.mmr_store_reload(self._h, s._h))
+
+    def IsOffloaded(self, store: StoreHandle) -> bool:
+        out = C.c_int32()
+        B.check(self._lib.mmr_store_is_offloaded(store._h, C.byref(out)))
+        return bool(out.value)
+
+    def PrepareReshard(self, srcs, dsts) -> None:
+        """Build and upload the plan of descriptor pair(s) before any store exists."""
+        if isinstance(srcs, B.ShardedShape):
+            srcs, dsts = [srcs], [dsts]
+        B.check(self._lib.mmr_context_prepare(self._h, _shape_array(srcs), _shape_array(dsts), len(srcs)))
+
     def SliceLocalShard(self, device: int, store: StoreHandle, wait: bool = True) -> int:
         p = C.c_void_p()
         fn = self._lib.mmr_store_shard_ptr if wait else self._lib.mmr_store_shard_ptr_async

@@ -57,10 +57,15 @@ struct mmr_store {
   mmr_sharded_shape shape{};
   mmr::Side side;
   std::string shape_key;
-  char* base = nullptr;   // one allocation, tile k at base + k * pitch
+  char* base = nullptr;   // one allocation, tile k at base + k * pitch (null for adopted stores)
   size_t pitch = 0;
   size_t bytes = 0;
+  std::vector<char*> adopted;  // caller-owned buffers, one per device (mmr_store_adopt)
+  char* host = nullptr;        // pinned host copy while the store is offloaded (the device buffers are gone then)
   mmr_context* owner = nullptr;
+
+  bool offloaded() const { return host != nullptr; }
+  char* tile(int64_t k) const { return adopted.empty() ? base + static_cast<size_t>(k) * pitch : adopted[static_cast<size_t>(k)]; }
 };
 
 struct mmr_context {
@@ -157,6 +162,10 @@ int reshard_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* d
     if (int rc = check_store(ctx, srcs[a], "source")) return rc;
     if (int rc = check_store(ctx, dsts[a], "destination")) return rc;
     if (srcs[a] == dsts[a]) return fail(MMR_INVALID_ARGUMENT, "array %d: source and destination are the same store", a);
+    // the mock's invariant (mm_mock_mm_xla.cc:164-173, 347-356): an offloaded store cannot take part in device work
+    if (srcs[a]->offloaded() || dsts[a]->offloaded())
+      return fail(MMR_INVALID_ARGUMENT, "array %d: store %lld is still offloaded to host memory", a,
+                  (long long)(srcs[a]->offloaded() ? srcs[a]->id : dsts[a]->id));
     ids.push_back(srcs[a]->id);
   }
   for (int a = 0; a < n; ++a) ids.push_back(dsts[a]->id);
@@ -183,8 +192,8 @@ int reshard_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* d
     std::vector<void*> ptrs(static_cast<size_t>(dp->plan.n_slots));
     for (int a = 0; a < n; ++a) {
       size_t slot = static_cast<size_t>(dp->plan.slot_bases[a]);
-      for (int64_t k = 0; k < srcs[a]->side.dev_count; ++k) ptrs[slot++] = srcs[a]->base + k * srcs[a]->pitch;
-      for (int64_t k = 0; k < dsts[a]->side.dev_count; ++k) ptrs[slot++] = dsts[a]->base + k * dsts[a]->pitch;
+      for (int64_t k = 0; k < srcs[a]->side.dev_count; ++k) ptrs[slot++] = srcs[a]->tile(k);
+      for (int64_t k = 0; k < dsts[a]->side.dev_count; ++k) ptrs[slot++] = dsts[a]->tile(k);
     }
     auto b = std::make_unique<Binding>();
     b->plan = dp;
@@ -256,7 +265,10 @@ void mmr_context_destroy(mmr_context* ctx) {
     (void)hipFree(p.second->d_generic);
     (void)hipFree(p.second->d_transposes);
   }
-  for (auto& s : ctx->stores) (void)hipFree(s.second->base);
+  for (auto& s : ctx->stores) {
+    (void)hipFree(s.second->base);
+    if (s.second->host) (void)hipHostFree(s.second->host);
+  }
   for (auto& c : ctx->buffer_cache)
     for (auto& b : c.second) (void)hipFree(b.base);
   (void)hipEventDestroy(ctx->t0);
@@ -322,7 +334,13 @@ int mmr_store_free(mmr_context* ctx, mmr_store* store, int32_t keep_in_cache) {
   if (int rc = check_store(ctx, store, "freed")) return rc;
   if (int rc = use_device(ctx)) return rc;
   drop_bindings_of(ctx, store->id);
-  if (keep_in_cache) {
+  if (store->host) {
+    MMR_HIP(hipHostFree(store->host));
+    ctx->stats.host_bytes_allocated -= static_cast<int64_t>(store->bytes);
+  } else if (!store->adopted.empty()) {
+    // caller-owned buffers: in-flight work on them must finish before the caller may reuse them
+    MMR_HIP(hipStreamSynchronize(ctx->stream));
+  } else if (keep_in_cache) {
     ctx->buffer_cache[store->shape_key].push_back(CachedBuffer{store->base, store->bytes});
   } else {
     MMR_HIP(hipFree(store->base));
@@ -365,7 +383,8 @@ int mmr_store_assemble(mmr_context* ctx, mmr_store* store, int64_t device, const
   const hipMemcpyKind kind = data_on_device == 1   ? hipMemcpyDeviceToDevice
                              : data_on_device == 0 ? hipMemcpyHostToDevice
                                                    : hipMemcpyDefault;  // the runtime looks the pointer up
-  MMR_HIP(hipMemcpyAsync(store->base + k * store->pitch, data, size, kind, ctx->stream));
+  if (store->offloaded()) return fail(MMR_INVALID_ARGUMENT, "store %lld is offloaded to host memory", (long long)store->id);
+  MMR_HIP(hipMemcpyAsync(store->tile(k), data, size, kind, ctx->stream));
   if (data_on_device != 1) MMR_HIP(hipStreamSynchronize(ctx->stream));  // host data is consumed before returning
   return MMR_OK;
 }
@@ -376,7 +395,8 @@ int mmr_store_shard_ptr_async(mmr_context* ctx, mmr_store* store, int64_t device
   if (int rc = check_store(ctx, store, "sliced")) return rc;
   int64_t k = 0;
   if (int rc = tile_index(store, device, &k)) return rc;
-  *ptr = store->base + k * store->pitch;
+  if (store->offloaded()) return fail(MMR_INVALID_ARGUMENT, "store %lld is offloaded to host memory", (long long)store->id);
+  *ptr = store->tile(k);
   return MMR_OK;
 }
 
@@ -395,7 +415,12 @@ int mmr_store_read_shard(mmr_context* ctx, mmr_store* store, int64_t device, voi
     return fail(MMR_INVALID_ARGUMENT, "read of %zu bytes exceeds the %lld-byte shard", size,
                 (long long)store->side.shard_bytes);
   if (int rc = use_device(ctx)) return rc;
-  if (size) MMR_HIP(hipMemcpyAsync(host_dst, store->base + k * store->pitch, size, hipMemcpyDeviceToHost, ctx->stream));
+  if (store->offloaded()) {
+    MMR_HIP(hipStreamSynchronize(ctx->stream));
+    std::memcpy(host_dst, store->host + static_cast<size_t>(k) * store->pitch, size);
+    return MMR_OK;
+  }
+  if (size) MMR_HIP(hipMemcpyAsync(host_dst, store->tile(k), size, hipMemcpyDeviceToHost, ctx->stream));
   MMR_HIP(hipStreamSynchronize(ctx->stream));
   return MMR_OK;
 }
@@ -414,6 +439,95 @@ int mmr_store_get_shape(const mmr_store* store, mmr_sharded_shape* out) {
 }
 
 int64_t mmr_store_id(const mmr_store* store) { return store ? store->id : -1; }
+
+int mmr_store_adopt(mmr_context* ctx, const mmr_sharded_shape* shape, const char* name, void* const* device_ptrs,
+                    mmr_store** out) {
+  if (!ctx || !shape || !out || !device_ptrs) return fail(MMR_INVALID_ARGUMENT, "null argument");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  auto s = std::make_unique<mmr_store>();
+  if (int rc = mmr::make_side(*shape, &s->side)) return rc;
+  for (int64_t k = 0; k < s->side.dev_count; ++k) {
+    if (!device_ptrs[k] && s->side.shard_bytes > 0) return fail(MMR_INVALID_ARGUMENT, "buffer of device %lld is null", (long long)(s->side.dev_start + k));
+    if (reinterpret_cast<uintptr_t>(device_ptrs[k]) % 16)
+      return fail(MMR_INVALID_ARGUMENT, "buffer of device %lld is not 16-byte aligned", (long long)(s->side.dev_start + k));
+    s->adopted.push_back(static_cast<char*>(device_ptrs[k]));
+  }
+  s->shape = *shape;
+  s->shape_key = mmr::descriptor_key(*shape);
+  s->name = name ? name : "anonymous";
+  s->owner = ctx;
+  s->pitch = static_cast<size_t>(s->side.shard_bytes);
+  s->bytes = 0;
+  s->id = g_next_store_id.fetch_add(1);
+  ctx->stats.stores_live += 1;
+  *out = s.get();
+  ctx->stores.emplace(s->id, std::move(s));
+  return MMR_OK;
+}
+
+int mmr_store_offload(mmr_context* ctx, mmr_store* store) {
+  if (!ctx) return fail(MMR_INVALID_ARGUMENT, "null context");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  if (int rc = check_store(ctx, store, "offloaded")) return rc;
+  if (store->offloaded()) return MMR_OK;
+  if (!store->adopted.empty()) return fail(MMR_INVALID_ARGUMENT, "store %lld lives in caller-owned buffers", (long long)store->id);
+  if (int rc = use_device(ctx)) return rc;
+  // pinned host memory is allocated, never registered after the fact
+  MMR_HIP(hipHostMalloc(reinterpret_cast<void**>(&store->host), store->bytes, hipHostMallocDefault));
+  MMR_HIP(hipMemcpyAsync(store->host, store->base, store->bytes, hipMemcpyDeviceToHost, ctx->stream));
+  MMR_HIP(hipStreamSynchronize(ctx->stream));
+  drop_bindings_of(ctx, store->id);
+  MMR_HIP(hipFree(store->base));
+  store->base = nullptr;
+  ctx->stats.bytes_allocated -= static_cast<int64_t>(store->bytes);
+  ctx->stats.host_bytes_allocated += static_cast<int64_t>(store->bytes);
+  ctx->stats.host_bytes_high_watermark = std::max(ctx->stats.host_bytes_high_watermark, ctx->stats.host_bytes_allocated);
+  return MMR_OK;
+}
+
+int mmr_store_reload(mmr_context* ctx, mmr_store* store) {
+  if (!ctx) return fail(MMR_INVALID_ARGUMENT, "null context");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  if (int rc = check_store(ctx, store, "reloaded")) return rc;
+  if (!store->offloaded()) return MMR_OK;
+  if (int rc = use_device(ctx)) return rc;
+  MMR_HIP(hipMalloc(reinterpret_cast<void**>(&store->base), store->bytes));
+  account_alloc(ctx, static_cast<int64_t>(store->bytes));
+  MMR_HIP(hipMemcpyAsync(store->base, store->host, store->bytes, hipMemcpyHostToDevice, ctx->stream));
+  MMR_HIP(hipStreamSynchronize(ctx->stream));  // the pinned buffer is released right away
+  MMR_HIP(hipHostFree(store->host));
+  store->host = nullptr;
+  ctx->stats.host_bytes_allocated -= static_cast<int64_t>(store->bytes);
+  return MMR_OK;
+}
+
+int mmr_store_is_offloaded(const mmr_store* store, int32_t* out) {
+  if (!store || !out) return fail(MMR_INVALID_ARGUMENT, "null argument");
+  *out = store->offloaded();
+  return MMR_OK;
+}
+
+int mmr_context_prepare(mmr_context* ctx, const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int32_t n) {
+  if (!ctx || n < 0 || (n > 0 && (!srcs || !dsts))) return fail(MMR_INVALID_ARGUMENT, "bad arguments");
+  if (n == 0) return MMR_OK;
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  if (int rc = use_device(ctx)) return rc;
+  std::vector<mmr_sharded_shape> s(srcs, srcs + n), d(dsts, dsts + n);
+  DevicePlan* dp = nullptr;
+  return get_plan(ctx, s, d, &dp);
+}
+
+int mmr_context_wait_event(mmr_context* ctx, void* hip_event) {
+  if (!ctx || !hip_event) return fail(MMR_INVALID_ARGUMENT, "null argument");
+  MMR_HIP(hipStreamWaitEvent(ctx->stream, static_cast<hipEvent_t>(hip_event), 0));
+  return MMR_OK;
+}
+
+int mmr_context_record_event(mmr_context* ctx, void* hip_event) {
+  if (!ctx || !hip_event) return fail(MMR_INVALID_ARGUMENT, "null argument");
+  MMR_HIP(hipEventRecord(static_cast<hipEvent_t>(hip_event), ctx->stream));
+  return MMR_OK;
+}
 
 int mmr_reshard(mmr_context* ctx, mmr_store* src, mmr_store* dst) {
   if (!ctx) return fail(MMR_INVALID_ARGUMENT, "null context");

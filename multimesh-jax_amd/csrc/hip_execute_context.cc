@@ -233,6 +233,39 @@ void HipExecuteContext::Rename(StoreHandle& handle, std::string name) {
   if (handle.impl) handle.impl->name = std::move(name);
 }
 
+void HipExecuteContext::OffloadDtoH(int64_t local_device_id, const std::vector<StoreHandle>& to_offload,
+                                    const std::vector<StoreHandle>& pipelined, const std::string& task_name) {
+  (void)pipelined;
+  (void)task_name;
+  std::lock_guard<std::mutex> lock(mu_);
+  bool first = false;
+  const int64_t seq = next_seq_["OffloadDtoH"][local_device_id];
+  ReplicatedOp& op = Arrive("OffloadDtoH", local_device_id, &first);
+  if (first) {
+    for (const StoreHandle& h : to_offload) {
+      require_live(h, "OffloadDtoH");
+      check(mmr_store_offload(ctx_, h.impl->array->store), "OffloadDtoH");
+    }
+  }
+  Leave("OffloadDtoH", seq, op);
+}
+
+void HipExecuteContext::OffloadHtoD(int64_t local_device_id, const std::vector<StoreHandle>& to_offload,
+                                    const std::string& task_name) {
+  (void)task_name;
+  std::lock_guard<std::mutex> lock(mu_);
+  bool first = false;
+  const int64_t seq = next_seq_["OffloadHtoD"][local_device_id];
+  ReplicatedOp& op = Arrive("OffloadHtoD", local_device_id, &first);
+  if (first) {
+    for (const StoreHandle& h : to_offload) {
+      require_live(h, "OffloadHtoD");
+      check(mmr_store_reload(ctx_, h.impl->array->store), "OffloadHtoD");
+    }
+  }
+  Leave("OffloadHtoD", seq, op);
+}
+
 void HipExecuteContext::CloseWindow() {}
 
 void HipExecuteContext::RunAfterAllTasks(int64_t local_device_id, std::function<void()> on_done) {

@@ -152,6 +152,11 @@ class HipExecuteContext {
   void Destroy(StoreHandle& store);
   void ClearStoreCache(int64_t local_device_id);
   void Rename(StoreHandle& handle, std::string name);
+  // zuku_execute_context.h:61-68.  `pipelined` stores must have been produced
+  // before the offload starts; on one stream that already holds.
+  void OffloadDtoH(int64_t local_device_id, const std::vector<StoreHandle>& to_offload,
+                   const std::vector<StoreHandle>& pipelined, const std::string& task_name);
+  void OffloadHtoD(int64_t local_device_id, const std::vector<StoreHandle>& to_offload, const std::string& task_name);
 
   void OpenWindow() {}
   void CloseWindow();

@@ -139,6 +139,22 @@ static int run() {
   EXPECT(ctx->Stats().plans_built == 1);
   EXPECT(ctx->Stats().binding_cache_hits == 1);
 
+  // offload to pinned host memory and back, issued by every local device like any other op
+  {
+    const int64_t dev_bytes = ctx->Stats().bytes_allocated;
+    for (int d = 0; d < kLocal; ++d) ctx->OffloadDtoH(d, {root[d]}, {}, "task");
+    EXPECT(ctx->Stats().bytes_allocated < dev_bytes);
+    EXPECT(ctx->Stats().host_bytes_allocated > 0);
+    // the mock's invariant: an offloaded store cannot take part in device work
+    EXPECT(throws([&] { ctx->Reshard(0, 0, param[0], root[0]); }, "offloaded"));  // consumes no position
+    for (int d = 0; d < kLocal; ++d) ctx->OffloadHtoD(d, {root[d]}, "task");
+    EXPECT(ctx->Stats().bytes_allocated == dev_bytes);
+    EXPECT(ctx->Stats().host_bytes_allocated == 0);
+    std::vector<uint16_t> got(expect[0].size());
+    ctx->CopyShardToHost(root[8], got.data(), got.size() * 2);
+    EXPECT(std::memcmp(got.data(), expect[0].data(), got.size() * 2) == 0);
+  }
+
   // control replication broken: device 1 describes the k-th store differently from device 0
   {
     StoreHandle a = ctx->CreateStore(0, 0, dst);

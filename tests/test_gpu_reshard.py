@@ -302,3 +302,85 @@ def test_reshard_is_stream_ordered_after_assemble(ctx):
     ctx.SliceLocalShard(dsts[0].devices[0], dsts[0])  # blocks
     _compare([a], [g], [read_all(ctx, dsts[0])])
     ctx.Free(srcs[0]); ctx.Free(dsts[0])
+
+
+def test_adopted_buffers_are_used_in_place(ctx):
+    """Zero-copy import and export: stores living in caller-owned device buffers on either side."""
+    a = workloads.config(2, 8)[0]
+    g = workloads.generate(a)
+    s_shape, d_shape = lib_shape(a["type"], a["src"]), lib_shape(a["type"], a["dst"])
+    # "native" buffers: two ordinary stores stand in for memory another runtime owns
+    srcs, dsts = make_stores(ctx, [a], [g])
+    src_ptrs = [ctx.SliceLocalShard(d, srcs[0]) for d in srcs[0].devices]
+    dst_ptrs = [ctx.SliceLocalShard(d, dsts[0]) for d in dsts[0].devices]
+    before = ctx.stats["bytes_allocated"]
+    adopted_src = ctx.AdoptShards(s_shape, src_ptrs, name="native.in")
+    adopted_dst = ctx.AdoptShards(d_shape, dst_ptrs, name="native.out")
+    assert ctx.stats["bytes_allocated"] == before  # nothing was allocated or copied
+    assert ctx.SliceLocalShard(3, adopted_src) == src_ptrs[3]
+    ctx.Reshard(adopted_src, adopted_dst)
+    ctx.Sync()
+    _compare([a], [g], [read_all(ctx, dsts[0])])  # the result is in the caller's buffers
+    with pytest.raises(mm.MmrError):
+        ctx.AdoptShards(s_shape, [p + 2 for p in src_ptrs])  # misaligned
+    ctx.Free(adopted_src); ctx.Free(adopted_dst)
+    # the caller's buffers outlive the adopting stores
+    _compare([a], [g], [read_all(ctx, dsts[0])])
+    ctx.Free(srcs[0]); ctx.Free(dsts[0])
+
+
+def test_offload_to_host_and_back(ctx):
+    """OffloadDtoH / OffloadHtoD with pinned host memory; the mock's invariant that an
+    offloaded store cannot take part in device work (mm_mock_mm_xla.cc:347-356)."""
+    a = workloads.config(1, 8)[0]
+    g = workloads.generate(a)
+    srcs, dsts = make_stores(ctx, [a], [g])
+    s0 = ctx.stats
+    ctx.OffloadDtoH([srcs[0]])
+    s1 = ctx.stats
+    assert ctx.IsOffloaded(srcs[0])
+    assert s1["bytes_allocated"] < s0["bytes_allocated"]
+    assert s1["host_bytes_allocated"] == s0["bytes_allocated"] - s1["bytes_allocated"]
+    with pytest.raises(mm.MmrError) as e:
+        ctx.Reshard(srcs[0], dsts[0])
+    assert "offloaded" in str(e.value)
+    with pytest.raises(mm.MmrError):
+        ctx.SliceLocalShard(srcs[0].devices[0], srcs[0])
+    host_view = ctx.ReadShard(srcs[0], srcs[0].devices[1])  # reading back still works
+    ctx.OffloadHtoD([srcs[0]])
+    assert not ctx.IsOffloaded(srcs[0])
+    assert ctx.stats["host_bytes_allocated"] == 0 and ctx.stats["bytes_allocated"] == s0["bytes_allocated"]
+    assert ctx.ReadShard(srcs[0], srcs[0].devices[1]).tobytes() == host_view.tobytes()
+    ctx.Reshard(srcs[0], dsts[0])
+    ctx.Sync()
+    _compare([a], [g], [read_all(ctx, dsts[0])])
+    ctx.Free(srcs[0]); ctx.Free(dsts[0])
+
+
+def test_plan_prepared_before_the_first_reshard(ctx):
+    s_shape = mm.sharded_shape("F32", [(96, 3, 0), (160, 1, 1)], 0, 3)
+    d_shape = mm.sharded_shape("F32", [(96, 1, 0), (160, 5, 1)], 3, 5)
+    s0 = ctx.stats
+    ctx.PrepareReshard(s_shape, d_shape)
+    s1 = ctx.stats
+    assert s1["plans_built"] == s0["plans_built"] + 1
+    a, b = ctx.CreateStore(s_shape), ctx.CreateStore(d_shape)
+    ctx.Reshard(a, b)
+    ctx.Sync()
+    s2 = ctx.stats
+    assert s2["plans_built"] == s1["plans_built"] and s2["plan_cache_hits"] == s1["plan_cache_hits"] + 1
+    ctx.Free(a); ctx.Free(b)
+
+
+def test_event_ordering_entry_points(ctx):
+    """The context's stream can wait for and record a caller's HIP event."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so.7")  # the runtime the library already loaded
+    ev = C.c_void_p()
+    assert hip.hipEventCreate(C.byref(ev)) == 0
+    lib = mm.load()
+    mm._binding.check(lib.mmr_context_record_event(ctx._h, ev))
+    assert hip.hipEventSynchronize(ev) == 0
+    mm._binding.check(lib.mmr_context_wait_event(ctx._h, ev))
+    ctx.Sync()
+    assert hip.hipEventDestroy(ev) == 0
