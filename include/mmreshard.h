@@ -101,6 +101,18 @@ int mmr_logical_to_physical_sharding(const int32_t* axes_flat, const int32_t* ax
                                      int64_t dev_start, int64_t dev_count, const int64_t* mesh_dims,
                                      int32_t n_mesh, int32_t list_all_devices, mmr_op_sharding* out);
 
+/* LogicalShardingToOpSharding, mpmd_logical_to_gspmd_sharding.cc:21-124: the
+ * PartitionSpec-style logical axis names of one array, resolved through a
+ * task's options (mesh dims and axis names, ordered logical -> device axis
+ * pairs).  Tensor dim i carries the names spec_names[spec_begin[i] ..
+ * spec_begin[i+1]).  list_all_devices is dev_count < total_devices (:87-88).
+ * Shardings that do not divide the shape are rejected (:101-113). */
+int mmr_logical_sharding_to_op_sharding(const int64_t* mesh_dims, const char* const* mesh_axis_names, int32_t n_mesh,
+                                        const char* const* logical_names, const char* const* logical_device_axes,
+                                        int32_t n_logical_axes, const char* const* spec_names, const int32_t* spec_begin,
+                                        int32_t rank, const int64_t* shape, int64_t dev_start, int64_t dev_count,
+                                        int64_t total_devices, mmr_op_sharding* out);
+
 /* HloSharding::tile_assignment().array(): device id of every tile in row-major
  * tile order (what mm_sharding_test.cc:111-227 compares). Writes n entries. */
 int mmr_tile_assignment_devices(const mmr_op_sharding* s, int64_t* out, int64_t capacity, int64_t* n);

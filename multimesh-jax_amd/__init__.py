@@ -7,8 +7,9 @@ the reference's names for the path.
 from . import _binding
 from ._binding import LIB_PATH, MmrError, load  # noqa: F401
 from .api import (  # noqa: F401
-    CanonicalizeSharding, ComputeGlobalIndex, ComputeIndexSet, LogicalToPhysicalSharding,
+    CanonicalizeSharding, ComputeGlobalIndex, ComputeIndexSet, LogicalShardingToOpSharding, LogicalToPhysicalSharding,
     MeshEquivalentSharding, NeedsReshard, Plan, ReshardContext, StoreHandle, TileAssignmentDevices,
-    XlaShapeToZukuShape, describe, device_of_tile, itemsize, op_sharding, shard_bytes, shard_extents,
+    XlaShapeToZukuShape, describe, device_of_tile, itemsize, op_sharding, partition_spec_to_sharded_shape, shard_bytes,
+    shard_extents,
     sharded_shape, tile_of_device,
 )

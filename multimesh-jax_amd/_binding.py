@@ -107,6 +107,8 @@ PROTOTYPES = {
     "mmr_compute_index_set": (C.c_int, [I64, P(I64), I32, P(I64)]),
     "mmr_compute_global_index": (C.c_int, [P(I64), P(I64), I32, P(I64)]),
     "mmr_logical_to_physical_sharding": (C.c_int, [P(I32), P(I32), I32, I64, I64, P(I64), I32, I32, P(OpSharding)]),
+    "mmr_logical_sharding_to_op_sharding": (C.c_int, [P(I64), P(C.c_char_p), I32, P(C.c_char_p), P(C.c_char_p), I32,
+                                                      P(C.c_char_p), P(I32), I32, P(I64), I64, I64, I64, P(OpSharding)]),
     "mmr_tile_assignment_devices": (C.c_int, [P(OpSharding), P(I64), I64, P(I64)]),
     "mmr_canonicalize_sharding": (C.c_int, [P(OpSharding), P(I64), I32, I32, I32, P(ShardedShape)]),
     "mmr_xla_shape_to_sharded_shape": (C.c_int, [P(I64), I32, I32, I64, I64, P(OpSharding), I32, P(ShardedShape)]),

@@ -108,6 +108,39 @@ def LogicalToPhysicalSharding(logical_to_device_axes: Sequence[Sequence[int]], d
     return out
 
 
+def _strs(values: Sequence[str]):
+    return (C.c_char_p * max(len(values), 1))(*[v.encode() for v in values])
+
+
+def LogicalShardingToOpSharding(mesh_dims: Sequence[int], mesh_axes: Sequence[str],
+                                logical_axes: Sequence[Tuple[str, str]], logical_axis_names: Sequence[Sequence[str]],
+                                shape: Sequence[int], devices: Tuple[int, int], total_devices: int) -> B.OpSharding:
+    """PartitionSpec-style names of one array -> OpSharding (mpmd_logical_to_gspmd_sharding.cc:21-124)."""
+    flat: List[str] = []
+    begin = [0]
+    for names in logical_axis_names:
+        flat.extend(names)
+        begin.append(len(flat))
+    out = B.OpSharding()
+    B.check(B.load().mmr_logical_sharding_to_op_sharding(
+        _i64(mesh_dims), _strs(mesh_axes), len(mesh_dims), _strs([a for a, _ in logical_axes]),
+        _strs([b for _, b in logical_axes]), len(logical_axes), _strs(flat), (C.c_int32 * len(begin))(*begin),
+        len(logical_axis_names), _i64(shape), devices[0], devices[1], total_devices, C.byref(out)))
+    return out
+
+
+def partition_spec_to_sharded_shape(mesh: Sequence[Tuple[str, int]], spec: Sequence[Optional[str]],
+                                    shape: Sequence[int], element_type: str, devices: Tuple[int, int],
+                                    total_devices: Optional[int] = None) -> B.ShardedShape:
+    """A jax-style PartitionSpec on a named mesh -> the descriptor the reshard consumes:
+    LogicalShardingToOpSharding with every mesh axis as its own logical axis, then XlaShapeToZukuShape."""
+    axes = [n for n, _ in mesh]
+    op = LogicalShardingToOpSharding([s for _, s in mesh], axes, [(n, n) for n in axes],
+                                     [[p] if p else [] for p in spec], shape, devices,
+                                     total_devices if total_devices is not None else devices[1])
+    return XlaShapeToZukuShape(shape, element_type, devices, op, True)
+
+
 def TileAssignmentDevices(op: B.OpSharding) -> List[int]:
     n = 1
     for i in range(op.n_tile_dims):

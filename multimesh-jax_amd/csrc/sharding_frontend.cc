@@ -3,6 +3,7 @@
 // src/pjrt_client/mm_sharding.{h,cc} and mpmd_insert_reshard.cc:33-43 with the
 // XLA proto types flattened to the PODs of mmreshard.h.
 #include <algorithm>
+#include <cstring>
 #include <numeric>
 #include <vector>
 
@@ -243,6 +244,56 @@ int mmr_logical_to_physical_sharding(const int32_t* axes_flat, const int32_t* ax
   r.replicate_on_last_tile_dim = any_unused;
   r.iota_offset = dev_start;  // :270
   *out = r;
+  return MMR_OK;
+}
+
+int mmr_logical_sharding_to_op_sharding(const int64_t* mesh_dims, const char* const* mesh_axis_names, int32_t n_mesh,
+                                        const char* const* logical_names, const char* const* logical_device_axes,
+                                        int32_t n_logical_axes, const char* const* spec_names, const int32_t* spec_begin,
+                                        int32_t rank, const int64_t* shape, int64_t dev_start, int64_t dev_count,
+                                        int64_t total_devices, mmr_op_sharding* out) {
+  if (!out || n_mesh < 0 || n_mesh > MMR_MAX_DIMS || rank < 0 || rank > MMR_MAX_DIMS || n_logical_axes < 0 ||
+      (rank > 0 && (!spec_begin || !shape)))
+    return fail(MMR_INVALID_ARGUMENT, "bad arguments");
+  std::vector<std::vector<int32_t>> to_device(rank);
+  std::vector<int> used(n_mesh, 0);
+  std::vector<int64_t> sharding_on_axis(rank, 1);
+  for (int p = 0; p < n_logical_axes; ++p) {  // mpmd_logical_to_gspmd_sharding.cc:40-85, in the pairs' order
+    for (int idx = 0; idx < rank; ++idx) {
+      for (int k = spec_begin[idx]; k < spec_begin[idx + 1]; ++k) {
+        if (std::strcmp(spec_names[k], logical_names[p]) != 0) continue;
+        int di = -1;
+        for (int a = 0; a < n_mesh; ++a)
+          if (std::strcmp(mesh_axis_names[a], logical_device_axes[p]) == 0) {
+            di = a;
+            break;
+          }
+        if (di < 0) return fail(MMR_INVALID_ARGUMENT, "unknown device axis '%s' in autosharding", logical_device_axes[p]);
+        const int64_t total = sharding_on_axis[idx] * mesh_dims[di];
+        if (total <= shape[idx] && !used[di]) {
+          to_device[idx].push_back(di);
+          used[di] = 1;
+          sharding_on_axis[idx] = total;
+        }
+        break;
+      }
+    }
+  }
+  std::vector<int32_t> flat, begin{0};
+  for (auto& axes : to_device) {
+    flat.insert(flat.end(), axes.begin(), axes.end());
+    begin.push_back(static_cast<int32_t>(flat.size()));
+  }
+  const int32_t list_all = dev_count < total_devices;  // :87-88
+  if (int rc = mmr_logical_to_physical_sharding(flat.data(), begin.data(), rank, dev_start, dev_count, mesh_dims, n_mesh,
+                                                list_all, out))
+    return rc;
+  if (out->type == MMR_SHARDING_OTHER) {  // :101-113: the sharding must divide every dim
+    for (int d = 0; d < rank; ++d)
+      if (shape[d] % out->tile_dims[d])
+        return fail(MMR_INVALID_ARGUMENT, "sharding does not evenly divide shape: dim %d of extent %lld over %lld tiles", d,
+                    (long long)shape[d], (long long)out->tile_dims[d]);
+  }
   return MMR_OK;
 }
 

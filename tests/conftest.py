@@ -10,6 +10,15 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    # Tests load what is built; only when nothing is built do they build it (hipcc cross-compiles without a GPU).
+    import subprocess
+    if not os.path.exists(os.path.join(ROOT, "multimesh-jax_amd", "libmmreshard.so")):
+        subprocess.check_call(["bash", os.path.join(ROOT, "multimesh-jax_amd", "csrc", "build.sh")])
+    if not os.path.exists(os.path.join(ROOT, "oracle", "libreshard_oracle.so")):
+        subprocess.check_call(["make", "-s", "-C", os.path.join(ROOT, "oracle")])
+    if not (os.path.exists(os.path.join(ROOT, "tests", "cpp", "libmmr_emulation.so"))
+            and os.path.exists(os.path.join(ROOT, "tests", "cpp", "hip_execute_context_test"))):
+        subprocess.check_call(["bash", os.path.join(ROOT, "tests", "cpp", "build.sh")])
 
 
 @pytest.fixture(scope="session")

@@ -185,3 +185,64 @@ def test_raw_iota_shardings_agree_with_the_oracle(reshape_dims, data):
     got = mm.describe(mm.CanonicalizeSharding(lib_op, shape, "F32", True))
     assert got["dims"] == [[x.size, x.sharding, x.permutation] for x in expect.dims]
     assert n == got["dev_count"]
+
+
+def test_partition_specs_of_the_benchmark_configurations():
+    """BASELINE.json's (mesh, PartitionSpec) pairs give exactly the descriptors the workloads use."""
+    from multimesh_jax_amd import workloads
+    cases = [
+        (1, "src", [("x", 4)], ["x", None], (0, 4)),
+        (1, "dst", [("a", 2), ("b", 2)], ["a", "b"], (4, 4)),
+        (2, "src", [("t", 8)], [None, None, "t"], (0, 8)),
+        (2, "dst", [("s", 4)], [None, "s", None], (8, 4)),
+        (3, "src", [("h", 4), ("r", 2)], [None, "h", None, None], (0, 8)),
+        (3, "dst", [("s", 8)], [None, None, "s", None], (8, 8)),
+    ]
+    for index, side, mesh, spec, devices in cases:
+        a = workloads.config(index)[0]
+        ss = mm.partition_spec_to_sharded_shape(mesh, spec, a["shape"], a["type"], devices, total_devices=16)
+        got = mm.describe(ss)
+        assert [tuple(d) for d in got["dims"]] == [tuple(d) for d in a[side]["dims"]], (index, side)
+        assert (got["dev_start"], got["dev_count"]) == (a[side]["dev_start"], a[side]["dev_count"])
+
+
+def test_logical_sharding_rejects_non_divisible_and_unknown_axes():
+    # mpmd_logical_to_gspmd_sharding.cc:101-113
+    with pytest.raises(mm.MmrError) as e:
+        mm.LogicalShardingToOpSharding([3], ["x"], [("x", "x")], [[], ["x"]], [8, 4097], (0, 3), 3)
+    assert "evenly divide" in str(e.value)
+    with pytest.raises(so.ShardingError):
+        so.logical_sharding_to_op_sharding([3], ["x"], [("x", "x")], [[], ["x"]], [8, 4097], (0, 3), 3)
+    # :61-64
+    with pytest.raises(mm.MmrError) as e:
+        mm.LogicalShardingToOpSharding([4], ["x"], [("batch", "y")], [["batch"]], [8], (0, 4), 4)
+    assert "unknown device axis" in str(e.value)
+
+
+@given(st.data())
+@settings(max_examples=200, deadline=None)
+def test_logical_sharding_agrees_with_the_oracle(data):
+    mesh_axes = ["x", "y", "z"][:data.draw(st.integers(1, 3))]
+    mesh_dims = [data.draw(st.integers(1, 4)) for _ in mesh_axes]
+    logical_pool = ["batch", "seq", "hidden", "heads"]
+    pairs = [(l, data.draw(st.sampled_from(mesh_axes))) for l in logical_pool if data.draw(st.booleans())]
+    rank = data.draw(st.integers(0, 4))
+    names = [data.draw(st.lists(st.sampled_from(logical_pool), max_size=2, unique=True)) for _ in range(rank)]
+    shape = [data.draw(st.sampled_from([1, 2, 4, 6, 8, 12, 16])) for _ in range(rank)]
+    count = int(np.prod(mesh_dims))
+    start = data.draw(st.integers(0, 4))
+    total = count + data.draw(st.sampled_from([0, 0, 8]))
+    try:
+        expect = so.logical_sharding_to_op_sharding(mesh_dims, mesh_axes, pairs, names, shape, (start, count), total)
+    except so.ShardingError:
+        with pytest.raises(mm.MmrError):
+            mm.LogicalShardingToOpSharding(mesh_dims, mesh_axes, pairs, names, shape, (start, count), total)
+        return
+    got = _op_dict(mm.LogicalShardingToOpSharding(mesh_dims, mesh_axes, pairs, names, shape, (start, count), total))
+    assert got["type"] == expect.type
+    if expect.type == "OTHER":
+        assert got["tile_dims"] == expect.tile_assignment_dimensions
+        assert got["iota_reshape_dims"] == expect.iota_reshape_dims
+        assert got["iota_transpose_perm"] == expect.iota_transpose_perm
+        assert got["replicate_on_last_tile_dim"] == expect.replicate_on_last_tile_dim
+        assert got["iota_offset"] == expect.iota_offset
