@@ -28,7 +28,7 @@
 
 namespace mmr {
 
-struct V16 {
+struct alignas(16) V16 {
   uint32_t x, y, z, w;
 };
 
@@ -237,12 +237,21 @@ MMR_HD void generic_chunk(const mmr_copy_chunk& c, typename M::cptr src, typenam
 // byte, 32 for 16-byte elements.
 //
 // Vector path (tile 16-byte aligned on both sides, extents multiples of the
-// vector width): every global access is a 16-byte vector.  A lane loads one
-// vector of a source row, scatters its elements into LDS laid out [x][y] (row
-// pitch EDGE + elements-per-vector, so rows stay 16-byte aligned), and after the
-// barrier reads one 16-byte vector of an LDS row = consecutive y of one x and
-// stores it to the destination row x.  All loads of a thread are issued before
-// its first LDS write.
+// vector width): every global access is a 16-byte vector and every LDS access
+// at least a dword.  A lane loads the same vector of kPack = 4 / itemsize
+// adjacent source rows (one row for elements of 4 bytes and more), so for each
+// of the vector's x it holds kPack consecutive y: one dword (or one element of
+// 8 / 16 bytes), written to row x of an LDS tile laid out [x][y] without
+// padding.  After the barrier a lane reads one 16-byte group of an LDS row =
+// consecutive y of one x and stores it to destination row x.  All global loads
+// of a thread are issued before its first LDS write.
+//
+// LDS banks: rows are a multiple of 128 bytes apart, so the 16-byte groups of a
+// row are permuted by XOR with a function of x whose low three bits differ
+// between the 8 lanes that write the same y of 8 neighbouring vectors (and
+// between any 8 consecutive x): the dword writes of 32 lanes then fall into 32
+// different banks.  Reads are conflict-free by construction (8 consecutive
+// lanes read the 8 groups of one 128-byte row segment).
 //
 // Element path (anything else, e.g. ragged edge tiles): one element per lane,
 // LDS laid out [y][x] with pitch EDGE + 1.
@@ -250,18 +259,28 @@ MMR_HD void generic_chunk(const mmr_copy_chunk& c, typename M::cptr src, typenam
 template <int ITEM>
 struct TransposeTile {
   static constexpr int kEdge = ITEM == 1 ? 128 : (ITEM == 16 ? 32 : 64);
-  static constexpr int kVec = 16 / ITEM;           // elements per 16-byte vector
-  static constexpr int kPitch = kEdge + kVec;      // vector path, elements
-  static constexpr int kPitch1 = kEdge + 1;        // element path, elements
-  static constexpr int kLdsBytes = kEdge * kPitch * ITEM;
+  static constexpr int kVec = 16 / ITEM;                   // elements per 16-byte vector
+  static constexpr int kPack = ITEM >= 4 ? 1 : 4 / ITEM;   // source rows a lane packs into one LDS word
+  static constexpr int kRowBytes = kEdge * ITEM;           // vector path: bytes per LDS row (no padding)
+  static constexpr int kRowVecs = kEdge / kVec;            // 16-byte groups per row, source or destination
+  static constexpr int kRowPacks = kEdge / kPack;          // packed row groups per tile
+  static constexpr int kPitch1 = kEdge + 1;                // element path, elements
+  static constexpr int kLdsBytes = kEdge * kPitch1 * ITEM; // the element path's tile; the vector path's is smaller
 };
-constexpr int kTransposeLdsBytes = 64 * 66 * 8;  // the largest of TransposeTile<>::kLdsBytes (8-byte elements)
+constexpr int kTransposeLdsBytes = 64 * 65 * 8;  // the largest of TransposeTile<>::kLdsBytes (8-byte elements)
 
 MMR_HD bool transpose_is_vector(const mmr_transpose_chunk& c) {
   const uint32_t vec = 16u / c.itemsize;
   const uint64_t bits = c.src_off | c.dst_off | static_cast<uint64_t>(c.src_ystride) | static_cast<uint64_t>(c.dst_xstride) |
                         static_cast<uint64_t>(c.src_bstride) | static_cast<uint64_t>(c.dst_bstride);
   return (bits & 15u) == 0 && c.nx % vec == 0 && c.ny % vec == 0;
+}
+
+// XOR applied to the 16-byte group index of LDS row x.
+template <int ITEM>
+MMR_HD uint32_t transpose_swizzle(uint32_t x) {
+  constexpr uint32_t vec = TransposeTile<ITEM>::kVec;
+  return (vec == 1 ? x : (x ^ (x / vec))) & 7u;
 }
 
 template <typename T>
@@ -279,26 +298,54 @@ MMR_HD T element_of(const V16& v, int i) {
   }
 }
 
+// Task t of a phase -> (row index, 16-byte group within the row).  8
+// consecutive lanes take the 8 groups of one 128-byte row segment, the next 8
+// lanes the same segment of the next row; rows wider than 128 bytes are covered
+// segment after segment.  `rows` is the number of rows in the phase.
+MMR_HD void transpose_task(uint32_t t, uint32_t rows, uint32_t* row, uint32_t* group) {
+  const uint32_t r = t >> 3;
+  *group = (t & 7u) + ((r / rows) << 3);
+  *row = r % rows;
+}
+
 template <class M, typename T, int THREADS>
 MMR_HD void transpose_load_vec(const mmr_transpose_chunk& c, typename M::cptr src, uint32_t b, T* lds, uint32_t tid) {
   typedef TransposeTile<sizeof(T)> G;
-  constexpr int kRowVecs = G::kEdge / G::kVec;                // vectors per full source row of the tile
-  constexpr int kPerThread = G::kEdge * kRowVecs / THREADS;   // vectors per thread
+  constexpr int kTasks = G::kRowPacks * G::kRowVecs / THREADS;  // per thread
+  static_assert(kTasks >= 1 && G::kRowPacks * G::kRowVecs % THREADS == 0, "tile does not divide over the workgroup");
   typename M::cptr s = src + b * c.src_bstride;
-  V16 v[kPerThread];
+  uint8_t* tile = reinterpret_cast<uint8_t*>(lds);
+  V16 v[kTasks][G::kPack];
 #pragma unroll
-  for (int k = 0; k < kPerThread; ++k) {
-    const uint32_t vi = tid + k * THREADS;
-    const uint32_t y = vi / kRowVecs, xv = vi % kRowVecs;
-    if (y < c.ny && xv * G::kVec < c.nx) v[k] = M::load16(s + (y * c.src_ystride + static_cast<int64_t>(xv) * 16));
+  for (int k = 0; k < kTasks; ++k) {
+    uint32_t yg, xv;
+    transpose_task(tid + k * THREADS, G::kRowPacks, &yg, &xv);
+    if (yg * G::kPack < c.ny && xv * G::kVec < c.nx) {
+#pragma unroll
+      for (int p = 0; p < G::kPack; ++p)
+        v[k][p] = M::load16(s + ((yg * G::kPack + p) * c.src_ystride + static_cast<int64_t>(xv) * 16));
+    }
   }
 #pragma unroll
-  for (int k = 0; k < kPerThread; ++k) {
-    const uint32_t vi = tid + k * THREADS;
-    const uint32_t y = vi / kRowVecs, xv = vi % kRowVecs;
-    if (y < c.ny && xv * G::kVec < c.nx) {
+  for (int k = 0; k < kTasks; ++k) {
+    uint32_t yg, xv;
+    transpose_task(tid + k * THREADS, G::kRowPacks, &yg, &xv);
+    if (yg * G::kPack < c.ny && xv * G::kVec < c.nx) {
+      const uint32_t ybyte = yg * G::kPack * static_cast<uint32_t>(sizeof(T));  // byte of y within LDS row x
 #pragma unroll
-      for (int i = 0; i < G::kVec; ++i) lds[(xv * G::kVec + i) * G::kPitch + y] = element_of<T>(v[k], i);
+      for (int i = 0; i < G::kVec; ++i) {
+        const uint32_t x = xv * G::kVec + i;
+        uint8_t* at = tile + x * G::kRowBytes + (((ybyte >> 4) ^ transpose_swizzle<sizeof(T)>(x)) << 4) + (ybyte & 15u);
+        if constexpr (sizeof(T) >= 4) {
+          *reinterpret_cast<T*>(at) = element_of<T>(v[k][0], i);
+        } else {
+          uint32_t word = 0;
+#pragma unroll
+          for (int p = 0; p < G::kPack; ++p)
+            word |= static_cast<uint32_t>(element_of<T>(v[k][p], i)) << (8 * static_cast<int>(sizeof(T)) * p);
+          *reinterpret_cast<uint32_t*>(at) = word;
+        }
+      }
     }
   }
 }
@@ -306,17 +353,22 @@ MMR_HD void transpose_load_vec(const mmr_transpose_chunk& c, typename M::cptr sr
 template <class M, typename T, int THREADS>
 MMR_HD void transpose_store_vec(const mmr_transpose_chunk& c, typename M::ptr dst, uint32_t b, const T* lds, uint32_t tid) {
   typedef TransposeTile<sizeof(T)> G;
-  constexpr int kRowVecs = G::kEdge / G::kVec;  // vectors per full destination row of the tile
-  constexpr int kPerThread = G::kEdge * kRowVecs / THREADS;
+  constexpr int kTasks = G::kEdge * G::kRowVecs / THREADS;  // per thread
   typename M::ptr d = dst + b * c.dst_bstride;
+  const uint8_t* tile = reinterpret_cast<const uint8_t*>(lds);
+  V16 v[kTasks];
 #pragma unroll
-  for (int k = 0; k < kPerThread; ++k) {
-    const uint32_t vi = tid + k * THREADS;
-    const uint32_t x = vi / kRowVecs, yv = vi % kRowVecs;
-    if (x < c.nx && yv * G::kVec < c.ny) {
-      const V16 v = *reinterpret_cast<const V16*>(&lds[x * G::kPitch + yv * G::kVec]);  // 16-byte aligned by construction
-      M::store16(d + (x * c.dst_xstride + static_cast<int64_t>(yv) * 16), v);
-    }
+  for (int k = 0; k < kTasks; ++k) {
+    uint32_t x, yv;
+    transpose_task(tid + k * THREADS, G::kEdge, &x, &yv);
+    if (x < c.nx && yv * G::kVec < c.ny)
+      v[k] = *reinterpret_cast<const V16*>(tile + x * G::kRowBytes + ((yv ^ transpose_swizzle<sizeof(T)>(x)) << 4));
+  }
+#pragma unroll
+  for (int k = 0; k < kTasks; ++k) {
+    uint32_t x, yv;
+    transpose_task(tid + k * THREADS, G::kEdge, &x, &yv);
+    if (x < c.nx && yv * G::kVec < c.ny) M::store16(d + (x * c.dst_xstride + static_cast<int64_t>(yv) * 16), v[k]);
   }
 }
 

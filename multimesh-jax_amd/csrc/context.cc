@@ -34,7 +34,11 @@ struct DevicePlan {
   mmr_copy_chunk* d_copy16 = nullptr;
   mmr_copy_chunk* d_generic = nullptr;
   mmr_transpose_chunk* d_transposes = nullptr;
-  uint32_t max_transpose_itemsize = 1;
+  struct TransposeRun {
+    uint32_t itemsize;
+    int64_t begin, count;
+  };
+  std::vector<TransposeRun> transpose_runs;  // the table is sorted by itemsize; one launch per run
 };
 
 struct Binding {
@@ -139,8 +143,11 @@ int get_plan(mmr_context* ctx, const std::vector<mmr_sharded_shape>& srcs, const
   if (int rc = upload(ctx, dp->plan.copy16, &dp->d_copy16)) return rc;
   if (int rc = upload(ctx, dp->plan.generic, &dp->d_generic)) return rc;
   if (int rc = upload(ctx, dp->plan.transposes, &dp->d_transposes)) return rc;
-  for (const mmr_transpose_chunk& c : dp->plan.transposes)
-    dp->max_transpose_itemsize = std::max(dp->max_transpose_itemsize, c.itemsize);
+  const std::vector<mmr_transpose_chunk>& tr = dp->plan.transposes;
+  for (int64_t i = 0; i < static_cast<int64_t>(tr.size()); ++i) {
+    if (i == 0 || tr[i].itemsize != tr[i - 1].itemsize) dp->transpose_runs.push_back({tr[i].itemsize, i, 0});
+    dp->transpose_runs.back().count += 1;
+  }
   ctx->stats.plans_built += 1;
   *out = dp.get();
   ctx->plans.emplace(std::move(key), std::move(dp));
@@ -213,9 +220,10 @@ int reshard_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* d
   // generic chunks leave partial lines at run boundaries; neighbours merge them when they share an L2
   MMR_HIP(mmr::launch_copy_generic(dp->d_generic, static_cast<int64_t>(p.generic.size()), binding->d_ptrs, xm == 0 ? 2 : xm,
                                    ctx->stream));
-  MMR_HIP(mmr::launch_transpose(dp->d_transposes, static_cast<int64_t>(p.transposes.size()), binding->d_ptrs, xm,
-                                dp->max_transpose_itemsize, ctx->stream));
-  ctx->stats.kernel_launches += (p.copy16.empty() ? 0 : 1) + (p.generic.empty() ? 0 : 1) + (p.transposes.empty() ? 0 : 1);
+  for (const DevicePlan::TransposeRun& run : dp->transpose_runs)
+    MMR_HIP(mmr::launch_transpose(dp->d_transposes + run.begin, run.count, binding->d_ptrs, xm, run.itemsize, ctx->stream));
+  ctx->stats.kernel_launches +=
+      (p.copy16.empty() ? 0 : 1) + (p.generic.empty() ? 0 : 1) + static_cast<int64_t>(dp->transpose_runs.size());
   return MMR_OK;
 }
 

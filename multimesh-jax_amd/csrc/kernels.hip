@@ -115,24 +115,19 @@ __device__ __forceinline__ void transpose_tiles(const mmr_transpose_chunk& c, gc
   }
 }
 
+template <typename T>
 __global__ __launch_bounds__(kTransposeThreads) void mmr_transpose_kernel(const mmr_transpose_chunk* __restrict__ chunks,
                                                                           uint32_t n, void* const* __restrict__ ptrs,
                                                                           uint32_t xcd_group) {
-  // sized at launch for the widest element in the table (5 KiB for 1-byte up to
-  // 33 KiB for 8-byte elements), so narrow types keep full occupancy
-  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  // one instance per element width, each with the register and LDS budget of its own tile
+  // (16.1 KiB for 1- and 4-byte, 8.1 KiB for 2-byte, 32.5 KiB for 8-byte, 16.5 KiB for 16-byte elements)
+  __shared__ __attribute__((aligned(16))) uint8_t lds[TransposeTile<sizeof(T)>::kLdsBytes];
   const uint32_t ci = chunk_index(blockIdx.x, xcd_group);
   if (ci >= n) return;  // uniform over the workgroup: no barrier is skipped by part of it
   const mmr_transpose_chunk c = chunks[ci];
   gcchar* src = slot_base(ptrs, c.src_slot, c.src_off);
   gchar* dst = slot_base(ptrs, c.dst_slot, c.dst_off);
-  switch (c.itemsize) {  // wave-uniform
-    case 1: transpose_tiles<uint8_t>(c, src, dst, lds); break;
-    case 2: transpose_tiles<uint16_t>(c, src, dst, lds); break;
-    case 4: transpose_tiles<uint32_t>(c, src, dst, lds); break;
-    case 8: transpose_tiles<uint64_t>(c, src, dst, lds); break;
-    default: transpose_tiles<V16>(c, src, dst, lds); break;
-  }
+  transpose_tiles<T>(c, src, dst, lds);
 }
 
 hipError_t check_grid(int64_t n) { return (n < 0 || n > 0x7ff00000LL) ? hipErrorInvalidValue : hipSuccess; }
@@ -163,27 +158,27 @@ hipError_t launch_copy_generic(const mmr_copy_chunk* d_chunks, int64_t n, void* 
   return hipGetLastError();
 }
 
-size_t transpose_lds_bytes(uint32_t itemsize) {
-  switch (itemsize) {
-    case 1: return TransposeTile<1>::kLdsBytes;
-    case 2: return TransposeTile<2>::kLdsBytes;
-    case 4: return TransposeTile<4>::kLdsBytes;
-    case 8: return TransposeTile<8>::kLdsBytes;
-    default: return TransposeTile<16>::kLdsBytes;
-  }
+template <typename T>
+hipError_t launch_transpose_of(const mmr_transpose_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
+                               hipStream_t stream) {
+  const uint32_t group = xcd_group_of(n, xcd_mode);
+  hipLaunchKernelGGL(mmr_transpose_kernel<T>, dim3(grid_size(n, group)), dim3(kTransposeThreads), 0, stream, d_chunks,
+                     static_cast<uint32_t>(n), d_ptrs, group);
+  return hipGetLastError();
 }
 
 hipError_t launch_transpose(const mmr_transpose_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
-                            uint32_t max_itemsize, hipStream_t stream) {
+                            uint32_t itemsize, hipStream_t stream) {
   if (n == 0) return hipSuccess;
   if (hipError_t e = check_grid(n)) return e;
-  const uint32_t group = xcd_group_of(n, xcd_mode);
-  // the element path's [y][x] tile (pitch edge + 1) is never larger than the vector path's for the same type
-  size_t lds = 0;
-  for (uint32_t item = 1; item <= 16 && item <= max_itemsize; item *= 2) lds = std::max(lds, transpose_lds_bytes(item));
-  hipLaunchKernelGGL(mmr_transpose_kernel, dim3(grid_size(n, group)), dim3(kTransposeThreads), lds, stream, d_chunks,
-                     static_cast<uint32_t>(n), d_ptrs, group);
-  return hipGetLastError();
+  switch (itemsize) {
+    case 1: return launch_transpose_of<uint8_t>(d_chunks, n, d_ptrs, xcd_mode, stream);
+    case 2: return launch_transpose_of<uint16_t>(d_chunks, n, d_ptrs, xcd_mode, stream);
+    case 4: return launch_transpose_of<uint32_t>(d_chunks, n, d_ptrs, xcd_mode, stream);
+    case 8: return launch_transpose_of<uint64_t>(d_chunks, n, d_ptrs, xcd_mode, stream);
+    case 16: return launch_transpose_of<V16>(d_chunks, n, d_ptrs, xcd_mode, stream);
+    default: return hipErrorInvalidValue;
+  }
 }
 
 }  // namespace mmr

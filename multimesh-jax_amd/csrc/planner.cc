@@ -370,12 +370,25 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
     auto cmp = [&](const mmr_copy_chunk& a, const mmr_copy_chunk& b) { return key(a) < key(b); };
     std::stable_sort(plan->copy16.begin(), plan->copy16.end(), cmp);
     std::stable_sort(plan->generic.begin(), plan->generic.end(), cmp);
+    // Tiles: by destination in blocks of 8 x 8 tiles rather than row after row, so the workgroups in flight
+    // together cover a compact region with long contiguous pieces on the source side as well as on the
+    // destination side (measured +10 % over plain destination order).
+    auto tile_key = [](const mmr_transpose_chunk& c) {
+      const uint64_t pitch = c.dst_xstride > 0 ? static_cast<uint64_t>(c.dst_xstride) : 1;
+      const uint64_t edge = c.itemsize == 1 ? 2 * kTransposeTile : (c.itemsize == 16 ? kTransposeTile / 2 : kTransposeTile);
+      const uint64_t x = c.dst_off / pitch, y = c.dst_off % pitch;  // destination row, byte within it
+      return std::make_tuple(c.dst_slot, x / (8 * edge), y / (8 * edge * c.itemsize), x, y);
+    };
     std::stable_sort(plan->transposes.begin(), plan->transposes.end(),
-                     [order](const mmr_transpose_chunk& a, const mmr_transpose_chunk& b) {
-                       return order == 2 ? std::make_pair(a.dst_slot, a.dst_off) < std::make_pair(b.dst_slot, b.dst_off)
+                     [&](const mmr_transpose_chunk& a, const mmr_transpose_chunk& b) {
+                       return order == 2 ? tile_key(a) < tile_key(b)
                                          : std::make_pair(a.src_slot, a.src_off) < std::make_pair(b.src_slot, b.src_off);
                      });
   }
+  // one launch per element width (a narrow type's kernel keeps its own register and LDS budget): runs of equal
+  // itemsize, the order above kept inside each run
+  std::stable_sort(plan->transposes.begin(), plan->transposes.end(),
+                   [](const mmr_transpose_chunk& a, const mmr_transpose_chunk& b) { return a.itemsize < b.itemsize; });
   plan->stats.n_arrays = n;
   plan->stats.n_copy16_chunks = static_cast<int64_t>(plan->copy16.size());
   plan->stats.n_copy_generic_chunks = static_cast<int64_t>(plan->generic.size());
