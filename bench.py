@@ -107,6 +107,15 @@ def measure(ctx, mm, workloads, args, config, with_parity=True):
     wall_s = time.perf_counter() - t0
 
     plan = ctx.plan_stats(sets[0][0][0], sets[0][1][0]) if len(arrays) == 1 else None
+    # cold plan construction (host only, excluded from the steady-state figure: plans are cached per descriptor pair)
+    from helpers import lib_shape
+    src_shapes = [lib_shape(a["type"], a["src"]) for a in arrays]
+    dst_shapes = [lib_shape(a["type"], a["dst"]) for a in arrays]
+    tp = time.perf_counter()
+    cold = mm.Plan(src_shapes, dst_shapes, args.chunk_bytes, args.order, args.xcd_mode)
+    plan_build_ms = (time.perf_counter() - tp) * 1e3
+    table_bytes = cold.stats["table_bytes"]
+    del cold
     generic = plan is not None and plan["n_copy_generic_chunks"] > plan["n_copy16_chunks"]
     res = {
         "alg_bytes": alg_bytes,
@@ -116,6 +125,8 @@ def measure(ctx, mm, workloads, args, config, with_parity=True):
         "achieved": alg_bytes / (kernel_ms / args.steps * 1e-3) / 1e9,
         "launches": launches,
         "plan": plan,
+        "plan_build_ms": plan_build_ms,
+        "plan_table_bytes": table_bytes,
         "kernel": ("mmr_transpose_kernel" if plan is not None and plan["n_transpose_chunks"] > 0 else
                    "mmr_copy_generic_kernel" if generic or config in (5, 6) else "mmr_copy16_kernel"),
         "n_arrays": len(arrays),
@@ -184,7 +195,8 @@ def main():
                 + (" ... (%d arrays)" % len(arrays) if len(arrays) > 3 else "")),
             "source": arrays[0]["src"], "destination": arrays[0]["dst"],
             "algorithmic_bytes": res["alg_bytes"], "buffer_sets": res["sets"],
-            "plan": res["plan"], "pct_hbm_peak": round(100.0 * res["value"] / HBM_PEAK_GBS, 2),
+            "plan": res["plan"], "plan_build_ms_cold": round(res["plan_build_ms"], 3),
+            "plan_table_bytes": res["plan_table_bytes"], "pct_hbm_peak": round(100.0 * res["value"] / HBM_PEAK_GBS, 2),
         },
         "roofline": {
             "bound": "hbm", "achieved": round(res["achieved"], 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -213,7 +225,8 @@ def main():
             r, *_rest = measure(ctx, mm, workloads, args, c)
             others["config%d" % c] = {"GB/s": round(r["achieved"], 1), "frac_hbm_peak": round(r["achieved"] / HBM_PEAK_GBS, 4),
                                        "kernel_ms": round(r["kernel_ms"], 5), "algorithmic_bytes": r["alg_bytes"],
-                                       "launches_per_step": r["launches"], "kernel": r["kernel"]}
+                                       "launches_per_step": r["launches"], "kernel": r["kernel"],
+                                       "plan_build_ms_cold": round(r["plan_build_ms"], 3)}
             for s in _rest[2] + _rest[3]:
                 ctx.Free(s)
         result["all_configs"] = others

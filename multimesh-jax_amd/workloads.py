@@ -132,6 +132,26 @@ def algorithmic_bytes(arrays: Sequence[dict]) -> int:
     return total
 
 
+def fp8_e4m3fn_bits(x: np.ndarray) -> np.ndarray:
+    """float32 -> float8 e4m3fn bit patterns (1 sign, 4 exponent bits of bias 7, 3 mantissa bits, no infinity,
+    0x7f = NaN, largest finite 448), round to nearest even.  Same bits as torch's `.to(torch.float8_e4m3fn)`;
+    kept in NumPy so that processes driving the GPU never import torch."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    bits = x.view(np.uint32)
+    sign = ((bits >> np.uint32(24)) & np.uint32(0x80)).astype(np.uint8)
+    mag = bits & np.uint32(0x7FFFFFFF)
+    a = mag.view(np.float32)
+    # normal range (>= 2^-6): round the mantissa to 3 bits, ties to even; a carry runs into the exponent by itself
+    lsb = (mag >> np.uint32(20)) & np.uint32(1)
+    rounded = (mag + np.uint32(0x7FFFF) + lsb) >> np.uint32(20)          # exponent (8 bits) | mantissa (3 bits)
+    normal = rounded.astype(np.int64) - ((127 - 7) << 3)
+    # subnormal range (< 2^-6): multiples of 2^-9; rint rounds ties to even, 8 lands on the smallest normal
+    sub = np.rint(np.where(a < np.float32(1.0), a, np.float32(0.0)).astype(np.float64) * 512.0).astype(np.int64)
+    code = np.where(a < np.float32(2.0 ** -6), sub, normal)
+    code = np.where((code > 0x7E) | np.isnan(a), 0x7F, code)              # beyond 448 after rounding, or NaN
+    return (code.astype(np.uint8) | sign).reshape(x.shape)
+
+
 def _bf16_bits(x: np.ndarray) -> np.ndarray:
     """float32 -> bfloat16 bit patterns, round to nearest even."""
     u = x.astype(np.float32).view(np.uint32)
@@ -155,9 +175,7 @@ def generate(a: dict) -> np.ndarray:
     elif dist == "int32000":
         return rng.integers(0, 32000, size=shape, dtype=np.int32).view(np.uint32)
     elif dist == "fp8":
-        import torch
-        x = np.clip(rng.standard_normal(size=shape, dtype=np.float32), -448.0, 448.0)
-        return torch.from_numpy(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+        return fp8_e4m3fn_bits(np.clip(rng.standard_normal(size=shape, dtype=np.float32), -448.0, 448.0))
     else:
         raise ValueError(dist)
     if a["type"] == "BF16":

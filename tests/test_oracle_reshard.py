@@ -186,3 +186,30 @@ def test_random_pairs_numpy_c_and_brute_force_agree(p):
     for d in expect:
         assert got[d].tobytes() == expect[d].tobytes()
         assert expect[d].tobytes() == brute_force_dst(g, dst, d, dm).tobytes()
+
+
+def test_fp8_workload_bits_equal_torch_cast():
+    """The fp8-e4m3fn benchmark input is specified as a torch cast; the workload
+    generator does it in NumPy (GPU processes stay free of torch).  Same bits on
+    every representable value, every rounding midpoint and its float32
+    neighbours, the overflow edge (448 / 464 / 480), specials and 3M random draws."""
+    torch = pytest.importorskip("torch")
+    from multimesh_jax_amd.workloads import fp8_e4m3fn_bits
+
+    def cast(x):
+        return torch.from_numpy(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+
+    rng = np.random.default_rng(0)
+    every = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).to(torch.float32).numpy()
+    finite = np.sort(every[np.isfinite(every)])
+    mid = ((finite[:-1].astype(np.float64) + finite[1:]) / 2).astype(np.float32)
+    up, down = np.float32(np.inf), np.float32(-np.inf)
+    points = np.concatenate([finite, mid, np.nextafter(mid, up), np.nextafter(mid, down), np.nextafter(finite, up),
+                             np.nextafter(finite, down)]).astype(np.float32)
+    special = np.array([0.0, -0.0, 1e-10, -1e-10, 2 ** -10, 2 ** -9, 3 * 2 ** -10, 2 ** -6, 447.9, 448, 463.99, 464, 464.01,
+                        479.9, 480, 500, 1e9, np.inf, -np.inf, np.nan], dtype=np.float32)
+    draws = [np.clip(rng.standard_normal(1_000_000, dtype=np.float32), -448, 448),
+             rng.standard_normal(1_000_000, dtype=np.float32) * np.float32(0.01),
+             rng.standard_normal(1_000_000, dtype=np.float32) * np.float32(200)]
+    for x in [points, special] + draws:
+        assert np.array_equal(fp8_e4m3fn_bits(x), cast(x))
