@@ -130,10 +130,15 @@ MMR_HD void copy16_chunk(const mmr_copy_chunk& c, typename M::cptr src, typename
 // (the planner emits generic chunks with n2 == 1).  Each row is cut at the
 // 16-byte boundaries of its DESTINATION: a lane owns one aligned 16-byte slot,
 // loads the matching source bytes with one unaligned 16-byte load and writes
-// one aligned 16-byte store.  The at most two ragged slots at the ends of a row
-// hold 1..15 bytes, moved as 8/4/2/1-byte pieces (binary decomposition of the
-// length).  The pieces travel in one V16: .x/.y the 8-byte piece, .z the 4-byte
-// piece, .w the 2-byte piece (low half) and the 1-byte piece (bits 16-23).
+// one 16-byte store.  A slot cut off by a row end (the first and the last slot
+// of a row, in general) slides inwards until it lies inside the row: it still
+// moves 16 bytes, now at an unaligned destination address, and overlaps its
+// neighbour, which writes the same values to the shared bytes.  So every lane
+// runs the same two instructions and no access ever leaves its row.  Rows
+// narrower than 16 bytes have no room to slide: their 1..15 bytes move as
+// 8/4/2/1-byte pieces (binary decomposition of the length), carried in one V16:
+// .x/.y the 8-byte piece, .z the 4-byte piece, .w the 2-byte piece (low half)
+// and the 1-byte piece (bits 16-23).
 // ---------------------------------------------------------------------------
 template <class M>
 MMR_HD V16 load_ragged(typename M::cptr s, uint32_t len) {
@@ -159,8 +164,8 @@ MMR_HD void store_ragged(typename M::ptr d, uint32_t len, V16 v) {
   if (len & 1) M::template storeu<uint8_t>(d + o1, static_cast<uint8_t>(v.w >> 16));
 }
 
-// One (row, slot) of a generic chunk: phase 1 (all loads).
-template <class M>
+// One (row, slot) of a generic chunk: phase 1 (all loads).  WIDE: rows of at least 16 bytes.
+template <class M, bool WIDE>
 MMR_HD void generic_load(const mmr_copy_chunk& c, typename M::cptr src, typename M::ptr dst, bool fill, uint32_t row,
                          uint32_t slot, V16* v, typename M::ptr* dpos, int32_t* len) {
   typename M::ptr drow = dst + row * c.d1;
@@ -168,28 +173,35 @@ MMR_HD void generic_load(const mmr_copy_chunk& c, typename M::cptr src, typename
   const int32_t w = static_cast<int32_t>(c.w);
   const int32_t mis = static_cast<int32_t>(M::addr(drow) & 15u);
   const int32_t rel = static_cast<int32_t>(slot << 4) - mis;  // row-relative byte where this aligned slot starts
-  const int32_t lo = rel < 0 ? 0 : rel;
-  const int32_t hi = rel + 16 < w ? rel + 16 : w;
-  *len = hi - lo;
-  *dpos = drow + lo;
-  if (*len == 16) {
+  if constexpr (WIDE) {
+    if (rel >= w) {
+      *len = 0;
+      return;
+    }
+    const int32_t lo = rel < 0 ? 0 : (rel + 16 > w ? w - 16 : rel);
+    *len = 16;
+    *dpos = drow + lo;
     *v = fill ? V16{0, 0, 0, 0} : M::load16u(srow + lo);
-  } else if (*len > 0) {
-    *v = fill ? V16{0, 0, 0, 0} : load_ragged<M>(srow + lo, static_cast<uint32_t>(*len));
+  } else {
+    const int32_t lo = rel < 0 ? 0 : rel;
+    const int32_t hi = rel + 16 < w ? rel + 16 : w;
+    *len = hi - lo;
+    *dpos = drow + lo;
+    if (*len > 0) *v = fill ? V16{0, 0, 0, 0} : load_ragged<M>(srow + lo, static_cast<uint32_t>(*len));
   }
 }
 
-template <class M>
+template <class M, bool WIDE>
 MMR_HD void generic_store(typename M::ptr dpos, int32_t len, V16 v) {
-  if (len == 16) {
-    M::store16(dpos, v);
-  } else if (len > 0) {
-    store_ragged<M>(dpos, static_cast<uint32_t>(len), v);
+  if constexpr (WIDE) {
+    if (len != 0) M::template storeu<V16>(dpos, v);  // aligned except for the slots that slid inwards
+  } else {
+    if (len > 0) store_ragged<M>(dpos, static_cast<uint32_t>(len), v);
   }
 }
 
-template <class M, int THREADS, int UNROLL>
-MMR_HD void generic_chunk(const mmr_copy_chunk& c, typename M::cptr src, typename M::ptr dst, uint32_t tid) {
+template <class M, int THREADS, int UNROLL, bool WIDE>
+MMR_HD void generic_rows(const mmr_copy_chunk& c, typename M::cptr src, typename M::ptr dst, uint32_t tid) {
   const bool fill = c.src_slot == MMR_SLOT_FILL;
   const uint32_t slots = ((c.w + 15u) >> 4) + 1u;  // a row of w bytes touches at most this many aligned slots
   const uint32_t rows = c.n1;
@@ -203,10 +215,10 @@ MMR_HD void generic_chunk(const mmr_copy_chunk& c, typename M::cptr src, typenam
         for (int u = 0; u < UNROLL; ++u) {
           len[u] = 0;
           const uint32_t slot = s0 + u * THREADS;
-          if (slot < slots) generic_load<M>(c, src, dst, fill, row, slot, &v[u], &dpos[u], &len[u]);
+          if (slot < slots) generic_load<M, WIDE>(c, src, dst, fill, row, slot, &v[u], &dpos[u], &len[u]);
         }
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) generic_store<M>(dpos[u], len[u], v[u]);
+        for (int u = 0; u < UNROLL; ++u) generic_store<M, WIDE>(dpos[u], len[u], v[u]);
       }
     }
     return;
@@ -223,11 +235,17 @@ MMR_HD void generic_chunk(const mmr_copy_chunk& c, typename M::cptr src, typenam
     for (int u = 0; u < UNROLL; ++u) {
       len[u] = 0;
       const uint32_t row = row0 + u * R;
-      if (row < rows) generic_load<M>(c, src, dst, fill, row, slot, &v[u], &dpos[u], &len[u]);
+      if (row < rows) generic_load<M, WIDE>(c, src, dst, fill, row, slot, &v[u], &dpos[u], &len[u]);
     }
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) generic_store<M>(dpos[u], len[u], v[u]);
+    for (int u = 0; u < UNROLL; ++u) generic_store<M, WIDE>(dpos[u], len[u], v[u]);
   }
+}
+
+template <class M, int THREADS, int UNROLL>
+MMR_HD void generic_chunk(const mmr_copy_chunk& c, typename M::cptr src, typename M::ptr dst, uint32_t tid) {
+  if (c.w >= 16) generic_rows<M, THREADS, UNROLL, true>(c, src, dst, tid);  // uniform over the workgroup
+  else generic_rows<M, THREADS, UNROLL, false>(c, src, dst, tid);
 }
 
 // ---------------------------------------------------------------------------
