@@ -20,8 +20,8 @@
 
 #include "mmreshard.h"
 
-#if defined(__HIPCC__) || defined(__CUDACC__)
-#define MMR_HD __host__ __device__ __forceinline__
+#if defined(__HIP__)
+#define MMR_HD __host__ __device__ inline __attribute__((always_inline))
 #else
 #define MMR_HD inline
 #endif
@@ -249,20 +249,25 @@ MMR_HD void generic_chunk(const mmr_copy_chunk& c, typename M::cptr src, typenam
 }
 
 // ---------------------------------------------------------------------------
-// Tile transpose: x is contiguous in the source, y in the destination.  The
-// caller puts a workgroup barrier between the load and the store phase and
-// after the store phase.  Tile edge in elements: 128 for 1-byte, 64 for 2/4/8-
-// byte, 32 for 16-byte elements.
+// Tile transpose: x is contiguous in the source, y in the destination.
+//
+// A workgroup owns a tile of kTileX x kTileY elements, its waves one
+// kEX x kEY sub-tile each (kWX x kWY waves; for 1-byte elements all four waves
+// share one sub-tile).
 //
 // Vector path (tile 16-byte aligned on both sides, extents multiples of the
-// vector width): every global access is a 16-byte vector and every LDS access
-// at least a dword.  A lane loads the same vector of kPack = 4 / itemsize
-// adjacent source rows (one row for elements of 4 bytes and more), so for each
-// of the vector's x it holds kPack consecutive y: one dword (or one element of
-// 8 / 16 bytes), written to row x of an LDS tile laid out [x][y] without
-// padding.  After the barrier a lane reads one 16-byte group of an LDS row =
-// consecutive y of one x and stores it to destination row x.  All global loads
-// of a thread are issued before its first LDS write.
+// vector width): every wave works alone, on its own slice of LDS, so the only
+// synchronisation is between the lanes of a wave (the caller puts a wave-level
+// fence between the two phases; a workgroup barrier where waves share a
+// sub-tile).  Every global
+// access is a 16-byte vector and every LDS access at least a dword.  A lane
+// loads the same vector of kPack = 4 / itemsize adjacent source rows (one row
+// for elements of 4 bytes and more), so for each of the vector's x it holds
+// kPack consecutive y: one dword (or one element of 8 / 16 bytes), written to
+// row x of an LDS tile laid out [x][y] without padding.  In the second phase a
+// lane reads one 16-byte group of an LDS row = consecutive y of one x and
+// stores it to destination row x.  All global loads of a lane are issued before
+// its first LDS write.
 //
 // LDS banks: rows are a multiple of 128 bytes apart, so the 16-byte groups of a
 // row are permuted by XOR with a function of x whose low three bits differ
@@ -271,21 +276,50 @@ MMR_HD void generic_chunk(const mmr_copy_chunk& c, typename M::cptr src, typenam
 // different banks.  Reads are conflict-free by construction (8 consecutive
 // lanes read the 8 groups of one 128-byte row segment).
 //
-// Element path (anything else, e.g. ragged edge tiles): one element per lane,
-// LDS laid out [y][x] with pitch EDGE + 1.
+// Element path (anything else, e.g. ragged edge tiles): the whole workgroup
+// walks the sub-tiles one after the other, one element per lane, LDS laid out
+// [y][x] with pitch kEX + 1; the caller puts a workgroup barrier after each
+// phase.
 // ---------------------------------------------------------------------------
 template <int ITEM>
 struct TransposeTile {
-  static constexpr int kEdge = ITEM == 1 ? 128 : (ITEM == 16 ? 32 : 64);
-  static constexpr int kVec = 16 / ITEM;                   // elements per 16-byte vector
-  static constexpr int kPack = ITEM >= 4 ? 1 : 4 / ITEM;   // source rows a lane packs into one LDS word
-  static constexpr int kRowBytes = kEdge * ITEM;           // vector path: bytes per LDS row (no padding)
-  static constexpr int kRowVecs = kEdge / kVec;            // 16-byte groups per row, source or destination
-  static constexpr int kRowPacks = kEdge / kPack;          // packed row groups per tile
-  static constexpr int kPitch1 = kEdge + 1;                // element path, elements
-  static constexpr int kLdsBytes = kEdge * kPitch1 * ITEM; // the element path's tile; the vector path's is smaller
+  // wave sub-tile: 128 bytes (or more) wide on both sides, so every access of 8 lanes is a full 128-byte line
+  static constexpr int kEX = ITEM == 1 ? 128 : (ITEM == 2 ? 64 : 32);
+  static constexpr int kEY = ITEM == 1 ? 128 : (ITEM == 16 ? 16 : (ITEM == 8 ? 32 : 64));
+  // Sub-tiles per workgroup tile, and the threads that share one.  1-byte elements: the smallest sub-tile is
+  // already 16 KiB, too many registers for one wave, so the four waves of the workgroup share a single sub-tile
+  // (and synchronise with a workgroup barrier instead of a wave fence).
+  static constexpr int kWX = ITEM == 1 ? 1 : 2, kWY = kWX;
+  static constexpr int kWaves = kWX * kWY;                   // number of sub-tiles
+  static constexpr int kGroupThreads = ITEM == 1 ? 256 : 64; // threads per sub-tile
+  static constexpr int kThreads = kGroupThreads * kWaves;
+  static constexpr int kTileX = kEX * kWX, kTileY = kEY * kWY;
+  static constexpr int kVec = 16 / ITEM;                     // elements per 16-byte vector
+  static constexpr int kPack = ITEM >= 4 ? 1 : 4 / ITEM;     // source rows a lane packs into one LDS word
+  static constexpr int kRowBytes = kEY * ITEM;               // vector path: bytes per LDS row (no padding)
+  static constexpr int kSrcVecs = kEX / kVec;                // 16-byte groups per source row of a sub-tile
+  static constexpr int kDstVecs = kEY / kVec;                // 16-byte groups per destination row of a sub-tile
+  static constexpr int kRowPacks = kEY / kPack;              // packed source-row groups per sub-tile
+  static constexpr int kWaveLdsBytes = kEX * kEY * ITEM;     // vector path: one wave's slice
+  static constexpr int kPitch1 = kEX + 1;                    // element path, elements
+  static constexpr int kLdsBytes =
+      kWaveLdsBytes * kWaves > kEY * kPitch1 * ITEM ? kWaveLdsBytes * kWaves : kEY * kPitch1 * ITEM;
+  static_assert(kSrcVecs % 8 == 0 && kDstVecs % 8 == 0, "sub-tile rows must be whole 128-byte lines");
+  static_assert(kSrcVecs * kRowPacks % kGroupThreads == 0 && kEX * kDstVecs % kGroupThreads == 0,
+                "sub-tile must divide over its threads");
 };
-constexpr int kTransposeLdsBytes = 64 * 65 * 8;  // the largest of TransposeTile<>::kLdsBytes (8-byte elements)
+constexpr int kTransposeLdsBytes = 32 * 1024 + 1024;  // at least the largest TransposeTile<>::kLdsBytes
+
+// Workgroup tile extents in elements for an element width (the planner cuts boxes into these).
+inline void transpose_tile_extent(uint32_t itemsize, uint32_t* tile_x, uint32_t* tile_y) {
+  switch (itemsize) {
+    case 1: *tile_x = TransposeTile<1>::kTileX; *tile_y = TransposeTile<1>::kTileY; break;
+    case 2: *tile_x = TransposeTile<2>::kTileX; *tile_y = TransposeTile<2>::kTileY; break;
+    case 4: *tile_x = TransposeTile<4>::kTileX; *tile_y = TransposeTile<4>::kTileY; break;
+    case 8: *tile_x = TransposeTile<8>::kTileX; *tile_y = TransposeTile<8>::kTileY; break;
+    default: *tile_x = TransposeTile<16>::kTileX; *tile_y = TransposeTile<16>::kTileY; break;
+  }
+}
 
 MMR_HD bool transpose_is_vector(const mmr_transpose_chunk& c) {
   const uint32_t vec = 16u / c.itemsize;
@@ -316,7 +350,7 @@ MMR_HD T element_of(const V16& v, int i) {
   }
 }
 
-// Task t of a phase -> (row index, 16-byte group within the row).  8
+// Task t of a wave's phase -> (row index, 16-byte group within the row).  8
 // consecutive lanes take the 8 groups of one 128-byte row segment, the next 8
 // lanes the same segment of the next row; rows wider than 128 bytes are covered
 // segment after segment.  `rows` is the number of rows in the phase.
@@ -326,19 +360,30 @@ MMR_HD void transpose_task(uint32_t t, uint32_t rows, uint32_t* row, uint32_t* g
   *row = r % rows;
 }
 
-template <class M, typename T, int THREADS>
+// Origin of the sub-tile of wave `wave` inside the workgroup tile, in elements.
+template <int ITEM>
+MMR_HD void transpose_subtile(uint32_t wave, uint32_t* x0, uint32_t* y0) {
+  typedef TransposeTile<ITEM> G;
+  *x0 = (wave % G::kWX) * G::kEX;
+  *y0 = (wave / G::kWX) * G::kEY;
+}
+
+// Vector path, phase 1: global -> registers -> this wave's LDS slice.  tid = thread of the workgroup.
+template <class M, typename T>
 MMR_HD void transpose_load_vec(const mmr_transpose_chunk& c, typename M::cptr src, uint32_t b, T* lds, uint32_t tid) {
   typedef TransposeTile<sizeof(T)> G;
-  constexpr int kTasks = G::kRowPacks * G::kRowVecs / THREADS;  // per thread
-  static_assert(kTasks >= 1 && G::kRowPacks * G::kRowVecs % THREADS == 0, "tile does not divide over the workgroup");
-  typename M::cptr s = src + b * c.src_bstride;
-  uint8_t* tile = reinterpret_cast<uint8_t*>(lds);
+  constexpr int kTasks = G::kSrcVecs * G::kRowPacks / G::kGroupThreads;  // per lane
+  const uint32_t wave = tid / G::kGroupThreads, lane = tid % G::kGroupThreads;
+  uint32_t x0, y0;
+  transpose_subtile<sizeof(T)>(wave, &x0, &y0);
+  typename M::cptr s = src + (b * c.src_bstride + y0 * c.src_ystride + static_cast<int64_t>(x0) * static_cast<int64_t>(sizeof(T)));
+  uint8_t* tile = reinterpret_cast<uint8_t*>(lds) + wave * G::kWaveLdsBytes;
   V16 v[kTasks][G::kPack];
 #pragma unroll
   for (int k = 0; k < kTasks; ++k) {
     uint32_t yg, xv;
-    transpose_task(tid + k * THREADS, G::kRowPacks, &yg, &xv);
-    if (yg * G::kPack < c.ny && xv * G::kVec < c.nx) {
+    transpose_task(lane + k * G::kGroupThreads, G::kRowPacks, &yg, &xv);
+    if (y0 + yg * G::kPack < c.ny && x0 + xv * G::kVec < c.nx) {
 #pragma unroll
       for (int p = 0; p < G::kPack; ++p)
         v[k][p] = M::load16(s + ((yg * G::kPack + p) * c.src_ystride + static_cast<int64_t>(xv) * 16));
@@ -347,8 +392,8 @@ MMR_HD void transpose_load_vec(const mmr_transpose_chunk& c, typename M::cptr sr
 #pragma unroll
   for (int k = 0; k < kTasks; ++k) {
     uint32_t yg, xv;
-    transpose_task(tid + k * THREADS, G::kRowPacks, &yg, &xv);
-    if (yg * G::kPack < c.ny && xv * G::kVec < c.nx) {
+    transpose_task(lane + k * G::kGroupThreads, G::kRowPacks, &yg, &xv);
+    if (y0 + yg * G::kPack < c.ny && x0 + xv * G::kVec < c.nx) {
       const uint32_t ybyte = yg * G::kPack * static_cast<uint32_t>(sizeof(T));  // byte of y within LDS row x
 #pragma unroll
       for (int i = 0; i < G::kVec; ++i) {
@@ -368,47 +413,60 @@ MMR_HD void transpose_load_vec(const mmr_transpose_chunk& c, typename M::cptr sr
   }
 }
 
-template <class M, typename T, int THREADS>
+// Vector path, phase 2: this wave's LDS slice -> registers -> global.
+template <class M, typename T>
 MMR_HD void transpose_store_vec(const mmr_transpose_chunk& c, typename M::ptr dst, uint32_t b, const T* lds, uint32_t tid) {
   typedef TransposeTile<sizeof(T)> G;
-  constexpr int kTasks = G::kEdge * G::kRowVecs / THREADS;  // per thread
-  typename M::ptr d = dst + b * c.dst_bstride;
-  const uint8_t* tile = reinterpret_cast<const uint8_t*>(lds);
+  constexpr int kTasks = G::kEX * G::kDstVecs / G::kGroupThreads;  // per lane
+  const uint32_t wave = tid / G::kGroupThreads, lane = tid % G::kGroupThreads;
+  uint32_t x0, y0;
+  transpose_subtile<sizeof(T)>(wave, &x0, &y0);
+  typename M::ptr d = dst + (b * c.dst_bstride + x0 * c.dst_xstride + static_cast<int64_t>(y0) * static_cast<int64_t>(sizeof(T)));
+  const uint8_t* tile = reinterpret_cast<const uint8_t*>(lds) + wave * G::kWaveLdsBytes;
   V16 v[kTasks];
 #pragma unroll
   for (int k = 0; k < kTasks; ++k) {
     uint32_t x, yv;
-    transpose_task(tid + k * THREADS, G::kEdge, &x, &yv);
-    if (x < c.nx && yv * G::kVec < c.ny)
+    transpose_task(lane + k * G::kGroupThreads, G::kEX, &x, &yv);
+    if (x0 + x < c.nx && y0 + yv * G::kVec < c.ny)
       v[k] = *reinterpret_cast<const V16*>(tile + x * G::kRowBytes + ((yv ^ transpose_swizzle<sizeof(T)>(x)) << 4));
   }
 #pragma unroll
   for (int k = 0; k < kTasks; ++k) {
     uint32_t x, yv;
-    transpose_task(tid + k * THREADS, G::kEdge, &x, &yv);
-    if (x < c.nx && yv * G::kVec < c.ny) M::store16(d + (x * c.dst_xstride + static_cast<int64_t>(yv) * 16), v[k]);
+    transpose_task(lane + k * G::kGroupThreads, G::kEX, &x, &yv);
+    if (x0 + x < c.nx && y0 + yv * G::kVec < c.ny) M::store16(d + (x * c.dst_xstride + static_cast<int64_t>(yv) * 16), v[k]);
   }
 }
 
-template <class M, typename T, int THREADS>
-MMR_HD void transpose_load(const mmr_transpose_chunk& c, typename M::cptr src, uint32_t b, T* lds, uint32_t tid) {
+// Element path: sub-tile `sub` of the workgroup tile, all threads of the workgroup.
+template <class M, typename T>
+MMR_HD void transpose_load(const mmr_transpose_chunk& c, typename M::cptr src, uint32_t b, uint32_t sub, T* lds, uint32_t tid) {
   typedef TransposeTile<sizeof(T)> G;
-  typename M::cptr s = src + b * c.src_bstride;
-  const uint32_t n = c.nx * c.ny;
-  for (uint32_t i = tid; i < n; i += THREADS) {
-    const uint32_t y = i / c.nx, x = i - y * c.nx;
+  uint32_t x0, y0;
+  transpose_subtile<sizeof(T)>(sub, &x0, &y0);
+  if (x0 >= c.nx || y0 >= c.ny) return;
+  const uint32_t nx = c.nx - x0 < G::kEX ? c.nx - x0 : G::kEX, ny = c.ny - y0 < G::kEY ? c.ny - y0 : G::kEY;
+  typename M::cptr s = src + (b * c.src_bstride + y0 * c.src_ystride + static_cast<int64_t>(x0) * static_cast<int64_t>(sizeof(T)));
+  const uint32_t n = nx * ny;
+  for (uint32_t i = tid; i < n; i += G::kThreads) {
+    const uint32_t y = i / nx, x = i - y * nx;
     lds[y * G::kPitch1 + x] =
         M::template loadu<T>(s + (y * c.src_ystride + static_cast<int64_t>(x) * static_cast<int64_t>(sizeof(T))));
   }
 }
 
-template <class M, typename T, int THREADS>
-MMR_HD void transpose_store(const mmr_transpose_chunk& c, typename M::ptr dst, uint32_t b, const T* lds, uint32_t tid) {
+template <class M, typename T>
+MMR_HD void transpose_store(const mmr_transpose_chunk& c, typename M::ptr dst, uint32_t b, uint32_t sub, const T* lds, uint32_t tid) {
   typedef TransposeTile<sizeof(T)> G;
-  typename M::ptr d = dst + b * c.dst_bstride;
-  const uint32_t n = c.nx * c.ny;
-  for (uint32_t i = tid; i < n; i += THREADS) {
-    const uint32_t x = i / c.ny, y = i - x * c.ny;
+  uint32_t x0, y0;
+  transpose_subtile<sizeof(T)>(sub, &x0, &y0);
+  if (x0 >= c.nx || y0 >= c.ny) return;
+  const uint32_t nx = c.nx - x0 < G::kEX ? c.nx - x0 : G::kEX, ny = c.ny - y0 < G::kEY ? c.ny - y0 : G::kEY;
+  typename M::ptr d = dst + (b * c.dst_bstride + x0 * c.dst_xstride + static_cast<int64_t>(y0) * static_cast<int64_t>(sizeof(T)));
+  const uint32_t n = nx * ny;
+  for (uint32_t i = tid; i < n; i += G::kThreads) {
+    const uint32_t x = i / ny, y = i - x * ny;
     M::template storeu<T>(d + (x * c.dst_xstride + static_cast<int64_t>(y) * static_cast<int64_t>(sizeof(T))),
                           lds[y * G::kPitch1 + x]);
   }

@@ -18,6 +18,7 @@
 #include <vector>
 
 #include "common.h"
+#include "chunk_ops.h"
 #include "kernels.h"
 #include "planner.h"
 
@@ -144,6 +145,14 @@ int get_plan(mmr_context* ctx, const std::vector<mmr_sharded_shape>& srcs, const
   if (int rc = upload(ctx, dp->plan.generic, &dp->d_generic)) return rc;
   if (int rc = upload(ctx, dp->plan.transposes, &dp->d_transposes)) return rc;
   const std::vector<mmr_transpose_chunk>& tr = dp->plan.transposes;
+  for (const mmr_transpose_chunk& c : tr) {  // the kernel's LDS tile and lane mapping assume these bounds
+    uint32_t tile_x = 0, tile_y = 0;
+    mmr::transpose_tile_extent(c.itemsize, &tile_x, &tile_y);
+    const bool width_ok = c.itemsize == 1 || c.itemsize == 2 || c.itemsize == 4 || c.itemsize == 8 || c.itemsize == 16;
+    if (!width_ok || c.nx == 0 || c.ny == 0 || c.nx > tile_x || c.ny > tile_y)
+      return fail(MMR_INTERNAL, "transpose chunk %u x %u of %u-byte elements does not fit the kernel's tile", c.nx, c.ny,
+                  c.itemsize);
+  }
   for (int64_t i = 0; i < static_cast<int64_t>(tr.size()); ++i) {
     if (i == 0 || tr[i].itemsize != tr[i - 1].itemsize) dp->transpose_runs.push_back({tr[i].itemsize, i, 0});
     dp->transpose_runs.back().count += 1;
@@ -223,7 +232,9 @@ int reshard_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* d
   MMR_HIP(mmr::launch_copy_generic(dp->d_generic, static_cast<int64_t>(p.generic.size()), binding->d_ptrs, generic_xm,
                                    ctx->stream));
   for (const DevicePlan::TransposeRun& run : dp->transpose_runs)
-    MMR_HIP(mmr::launch_transpose(dp->d_transposes + run.begin, run.count, binding->d_ptrs, xm, run.itemsize, ctx->stream));
+    // tiles are ordered in 8 x 8 blocks; runs of 64 table neighbours per XCD keep a block in one L2 (measured best)
+    MMR_HIP(mmr::launch_transpose(dp->d_transposes + run.begin, run.count, binding->d_ptrs, xm == 0 ? 64 : xm, run.itemsize,
+                                  ctx->stream));
   ctx->stats.kernel_launches +=
       (p.copy16.empty() ? 0 : 1) + (p.generic.empty() ? 0 : 1) + static_cast<int64_t>(dp->transpose_runs.size());
   return MMR_OK;

@@ -98,29 +98,55 @@ __global__ __launch_bounds__(THREADS) void mmr_copy_generic_kernel(const mmr_cop
   generic_chunk<DeviceMem<NTL, NTS>, THREADS, UNROLL>(c, src, dst, threadIdx.x);
 }
 
-constexpr int kTransposeThreads = 256;
+// Launch shape of the generic kernel (overridable at build time for tuning runs).
+#ifndef MMR_GENERIC_THREADS
+#define MMR_GENERIC_THREADS 256
+#endif
+#ifndef MMR_GENERIC_UNROLL
+#define MMR_GENERIC_UNROLL 2
+#endif
+#ifndef MMR_GENERIC_NT_LOADS
+#define MMR_GENERIC_NT_LOADS false
+#endif
+constexpr int kGenericThreads = MMR_GENERIC_THREADS;
+constexpr int kGenericUnroll = MMR_GENERIC_UNROLL;
+constexpr bool kGenericNtLoads = MMR_GENERIC_NT_LOADS;
+
+// Orders the LDS accesses of the lanes of one wave: what a lane wrote before is visible to the others after.
+__device__ __forceinline__ void wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
 
 template <typename T>
 __device__ __forceinline__ void transpose_tiles(const mmr_transpose_chunk& c, gcchar* src, gchar* dst, void* lds_raw) {
   typedef DeviceMem<true, true> M;
+  typedef TransposeTile<sizeof(T)> G;
   T* lds = static_cast<T*>(lds_raw);
-  const bool vec = transpose_is_vector(c);  // wave-uniform
+  if (transpose_is_vector(c)) {  // uniform over the workgroup; waves run independently
+    for (uint32_t b = 0; b < c.nb; ++b) {
+      transpose_load_vec<M, T>(c, src, b, lds, threadIdx.x);
+      if constexpr (G::kGroupThreads == 64) wave_sync(); else __syncthreads();
+      transpose_store_vec<M, T>(c, dst, b, lds, threadIdx.x);
+      if constexpr (G::kGroupThreads == 64) wave_sync(); else __syncthreads();
+    }
+    return;
+  }
   for (uint32_t b = 0; b < c.nb; ++b) {
-    if (vec) transpose_load_vec<M, T, kTransposeThreads>(c, src, b, lds, threadIdx.x);
-    else transpose_load<M, T, kTransposeThreads>(c, src, b, lds, threadIdx.x);
-    __syncthreads();
-    if (vec) transpose_store_vec<M, T, kTransposeThreads>(c, dst, b, lds, threadIdx.x);
-    else transpose_store<M, T, kTransposeThreads>(c, dst, b, lds, threadIdx.x);
-    __syncthreads();
+    for (uint32_t sub = 0; sub < G::kWaves; ++sub) {
+      transpose_load<M, T>(c, src, b, sub, lds, threadIdx.x);
+      __syncthreads();
+      transpose_store<M, T>(c, dst, b, sub, lds, threadIdx.x);
+      __syncthreads();
+    }
   }
 }
 
 template <typename T>
-__global__ __launch_bounds__(kTransposeThreads) void mmr_transpose_kernel(const mmr_transpose_chunk* __restrict__ chunks,
-                                                                          uint32_t n, void* const* __restrict__ ptrs,
-                                                                          uint32_t xcd_group) {
-  // one instance per element width, each with the register and LDS budget of its own tile
-  // (16.1 KiB for 1- and 4-byte, 8.1 KiB for 2-byte, 32.5 KiB for 8-byte, 16.5 KiB for 16-byte elements)
+__global__ __launch_bounds__(TransposeTile<sizeof(T)>::kThreads) void mmr_transpose_kernel(
+    const mmr_transpose_chunk* __restrict__ chunks, uint32_t n, void* const* __restrict__ ptrs, uint32_t xcd_group) {
+  // one instance per element width, each with the register and LDS budget of its own tile (32 KiB of LDS)
   __shared__ __attribute__((aligned(16))) uint8_t lds[TransposeTile<sizeof(T)>::kLdsBytes];
   const uint32_t ci = chunk_index(blockIdx.x, xcd_group);
   if (ci >= n) return;  // uniform over the workgroup: no barrier is skipped by part of it
@@ -153,8 +179,9 @@ hipError_t launch_copy_generic(const mmr_copy_chunk* d_chunks, int64_t n, void* 
   if (hipError_t e = check_grid(n)) return e;
   const uint32_t group = xcd_group_of(n, xcd_mode);
   // cacheable loads (a source line shared by two chunks is fetched once), nontemporal stores
-  hipLaunchKernelGGL((mmr_copy_generic_kernel<256, 2, false, true>), dim3(grid_size(n, group)), dim3(256), 0, stream,
-                     d_chunks, static_cast<uint32_t>(n), d_ptrs, group);
+  hipLaunchKernelGGL((mmr_copy_generic_kernel<kGenericThreads, kGenericUnroll, kGenericNtLoads, true>),
+                     dim3(grid_size(n, group)), dim3(kGenericThreads), 0, stream, d_chunks, static_cast<uint32_t>(n), d_ptrs,
+                     group);
   return hipGetLastError();
 }
 
@@ -162,8 +189,8 @@ template <typename T>
 hipError_t launch_transpose_of(const mmr_transpose_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
                                hipStream_t stream) {
   const uint32_t group = xcd_group_of(n, xcd_mode);
-  hipLaunchKernelGGL(mmr_transpose_kernel<T>, dim3(grid_size(n, group)), dim3(kTransposeThreads), 0, stream, d_chunks,
-                     static_cast<uint32_t>(n), d_ptrs, group);
+  hipLaunchKernelGGL(mmr_transpose_kernel<T>, dim3(grid_size(n, group)), dim3(TransposeTile<sizeof(T)>::kThreads), 0, stream,
+                     d_chunks, static_cast<uint32_t>(n), d_ptrs, group);
   return hipGetLastError();
 }
 

@@ -6,11 +6,13 @@
 // dropped, dims that are contiguous on both sides merged) and lowered to
 // workgroup-sized chunks:
 //   * copy chunks     - n2 x n1 rows of w contiguous bytes (minor dim kept),
-//   * transpose chunks - <=64x64-element tiles staged through LDS (source and
+//   * transpose chunks - workgroup tiles (128 x 128 elements for 2-byte types) staged through LDS (source and
 //                        destination disagree on the minor dim),
 //   * fill chunks      - copy chunks without a source, zeroing the pad of short
 //                        edge tiles.
 #include "planner.h"
+
+#include "chunk_ops.h"
 
 #include <algorithm>
 #include <cstring>
@@ -208,7 +210,9 @@ class Builder {
 
   void lower_transpose(uint32_t src_slot, uint32_t dst_slot, int64_t so, int64_t dof, const std::vector<BoxDim>& dims,
                        int x, int y, int itemsize) {
-    const int64_t tile = itemsize == 1 ? 2 * kTransposeTile : (itemsize == 16 ? kTransposeTile / 2 : kTransposeTile);
+    uint32_t tx = 0, ty = 0;
+    transpose_tile_extent(static_cast<uint32_t>(itemsize), &tx, &ty);
+    const int64_t tile_x = tx, tile_y = ty;
     const BoxDim dx = dims[x], dy = dims[y];
     std::vector<BoxDim> outer;
     for (int i = 0; i < static_cast<int>(dims.size()); ++i)
@@ -219,18 +223,20 @@ class Builder {
       db = outer[ib];
       outer.erase(outer.begin() + ib);
     }
-    const int64_t nb = std::max<int64_t>(1, std::min<int64_t>(db.n, chunk_bytes_ / (tile * tile * itemsize)));
+    // tiles narrower than the workgroup tile (a short x or y extent) are batched along the next dimension
+    const int64_t tile_bytes = std::min(tile_x, dx.n) * std::min(tile_y, dy.n) * itemsize;
+    const int64_t nb = std::max<int64_t>(1, std::min<int64_t>(db.n, kTransposeChunkBytes / tile_bytes));
     for_each_index(outer, [&](int64_t ds, int64_t dd) {
       for (int64_t b0 = 0; b0 < db.n; b0 += nb) {
-        for (int64_t y0 = 0; y0 < dy.n; y0 += tile) {
-          for (int64_t x0 = 0; x0 < dx.n; x0 += tile) {
+        for (int64_t y0 = 0; y0 < dy.n; y0 += tile_y) {
+          for (int64_t x0 = 0; x0 < dx.n; x0 += tile_x) {
             mmr_transpose_chunk c{};
             c.src_slot = src_slot;
             c.dst_slot = dst_slot;
             c.src_off = static_cast<uint64_t>(so + ds + b0 * db.s + y0 * dy.s + x0 * dx.s);
             c.dst_off = static_cast<uint64_t>(dof + dd + b0 * db.d + y0 * dy.d + x0 * dx.d);
-            c.nx = static_cast<uint32_t>(std::min(tile, dx.n - x0));
-            c.ny = static_cast<uint32_t>(std::min(tile, dy.n - y0));
+            c.nx = static_cast<uint32_t>(std::min(tile_x, dx.n - x0));
+            c.ny = static_cast<uint32_t>(std::min(tile_y, dy.n - y0));
             c.nb = static_cast<uint32_t>(std::min(nb, db.n - b0));
             c.itemsize = static_cast<uint32_t>(itemsize);
             c.src_ystride = dy.s;
@@ -389,9 +395,10 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
     // destination side (measured +10 % over plain destination order).
     auto tile_key = [](const mmr_transpose_chunk& c) {
       const uint64_t pitch = c.dst_xstride > 0 ? static_cast<uint64_t>(c.dst_xstride) : 1;
-      const uint64_t edge = c.itemsize == 1 ? 2 * kTransposeTile : (c.itemsize == 16 ? kTransposeTile / 2 : kTransposeTile);
+      uint32_t tx = 0, ty = 0;
+      transpose_tile_extent(c.itemsize, &tx, &ty);
       const uint64_t x = c.dst_off / pitch, y = c.dst_off % pitch;  // destination row, byte within it
-      return std::make_tuple(c.dst_slot, x / (8 * edge), y / (8 * edge * c.itemsize), x, y);
+      return std::make_tuple(c.dst_slot, x / (8ull * tx), y / (8ull * ty * c.itemsize), x, y);
     };
     std::stable_sort(plan->transposes.begin(), plan->transposes.end(),
                      [&](const mmr_transpose_chunk& a, const mmr_transpose_chunk& b) {

@@ -26,7 +26,7 @@ struct mmr_plan {
 namespace mmr {
 
 constexpr uint32_t kDefaultChunkBytes = 8 * 1024;
-constexpr uint32_t kTransposeTile = 64;  // elements per tile edge (128 for 1-byte, 32 for 16-byte elements)
+constexpr int64_t kTransposeChunkBytes = 32 * 1024;  // a transpose chunk batches small tiles up to this many bytes
 
 // Cache key of a batch of descriptor pairs under given options.
 std::string plan_key(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int n,

@@ -77,21 +77,22 @@ struct HostMem {
 
 template <typename T>
 void run_transpose(const mmr_transpose_chunk& c, const uint8_t* src, uint8_t* dst) {
-  constexpr int kThreads = 256;
+  typedef mmr::TransposeTile<sizeof(T)> G;
+  constexpr uint32_t kThreads = G::kThreads;
   alignas(16) static thread_local uint8_t lds_raw[mmr::kTransposeLdsBytes];
-  static_assert(mmr::TransposeTile<sizeof(T)>::kLdsBytes <= mmr::kTransposeLdsBytes, "LDS tile too large");
-  static_assert(mmr::TransposeTile<sizeof(T)>::kEdge * mmr::TransposeTile<sizeof(T)>::kPitch1 * sizeof(T) <=
-                    mmr::kTransposeLdsBytes, "LDS tile too large");
+  static_assert(G::kLdsBytes <= mmr::kTransposeLdsBytes, "LDS tile too large");
   T* lds = reinterpret_cast<T*>(lds_raw);
-  const bool vec = mmr::transpose_is_vector(c);
+  // a phase runs for every thread before the next one starts: what the wave fence (vector path) or the
+  // workgroup barrier (element path) guarantees on the device
   for (uint32_t b = 0; b < c.nb; ++b) {
-    for (uint32_t tid = 0; tid < kThreads; ++tid) {
-      if (vec) mmr::transpose_load_vec<HostMem, T, kThreads>(c, src, b, lds, tid);
-      else mmr::transpose_load<HostMem, T, kThreads>(c, src, b, lds, tid);
+    if (mmr::transpose_is_vector(c)) {
+      for (uint32_t tid = 0; tid < kThreads; ++tid) mmr::transpose_load_vec<HostMem, T>(c, src, b, lds, tid);
+      for (uint32_t tid = 0; tid < kThreads; ++tid) mmr::transpose_store_vec<HostMem, T>(c, dst, b, lds, tid);
+      continue;
     }
-    for (uint32_t tid = 0; tid < kThreads; ++tid) {
-      if (vec) mmr::transpose_store_vec<HostMem, T, kThreads>(c, dst, b, lds, tid);
-      else mmr::transpose_store<HostMem, T, kThreads>(c, dst, b, lds, tid);
+    for (uint32_t sub = 0; sub < G::kWaves; ++sub) {
+      for (uint32_t tid = 0; tid < kThreads; ++tid) mmr::transpose_load<HostMem, T>(c, src, b, sub, lds, tid);
+      for (uint32_t tid = 0; tid < kThreads; ++tid) mmr::transpose_store<HostMem, T>(c, dst, b, sub, lds, tid);
     }
   }
 }
@@ -192,8 +193,9 @@ int mmr_emulate_plan(const mmr_plan* plan, void* const* slot_ptrs, const size_t*
       }
       const uint8_t* src = base(c.src_slot, c.src_off);
       uint8_t* dst = base(c.dst_slot, c.dst_off);
-      const uint32_t tile = c.itemsize == 1 ? 128 : (c.itemsize == 16 ? 32 : 64);
-      if (c.nx > tile || c.ny > tile) {
+      uint32_t tile_x = 0, tile_y = 0;
+      mmr::transpose_tile_extent(c.itemsize, &tile_x, &tile_y);
+      if (c.nx > tile_x || c.ny > tile_y) {
         g_error = "transpose tile larger than the LDS tile";
         return;
       }
