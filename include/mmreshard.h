@@ -295,6 +295,14 @@ int mmr_reshard(mmr_context* ctx, mmr_store* src, mmr_store* dst);
  * class (the reference issues one Reshard call per array,
  * mm_pjrt_executable.cc:616-658). */
 int mmr_reshard_batch(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int32_t n);
+/* Everything mmr_reshard_batch does for these stores except the launches: the plan
+ * and the table of shard pointers are built, uploaded and cached, so that the next
+ * mmr_reshard / mmr_reshard_batch of the same stores only launches kernels and can
+ * be recorded into a HIP graph (stream capture forbids the allocations and copies
+ * of a first use; a reshard that would need them while the stream is capturing
+ * fails with MMR_INVALID_ARGUMENT and leaves the capture intact).  Schedule-build
+ * time work like MpmdScheduler::AddReshardTask, mpmd_partition.cc:340-351. */
+int mmr_reshard_bind(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int32_t n);
 
 /* Build and upload the plan of n descriptor pairs (one batch) ahead of the first
  * reshard, i.e. when the schedule entry is created (MpmdScheduler::AddReshardTask,

@@ -364,6 +364,16 @@ class ReshardContext:
             srcs, dsts = [srcs], [dsts]
         B.check(self._lib.mmr_context_prepare(self._h, _shape_array(srcs), _shape_array(dsts), len(srcs)))
 
+    def BindReshard(self, srcs, dsts) -> None:
+        """Plan and pointer table of these stores, built and uploaded without launching: the next
+        Reshard / ReshardBatch of the same stores only launches kernels (and may be captured into a HIP graph)."""
+        if isinstance(srcs, StoreHandle):
+            srcs, dsts = [srcs], [dsts]
+        n = len(srcs)
+        sa = (C.c_void_p * max(n, 1))(*[s._h for s in srcs])
+        da = (C.c_void_p * max(n, 1))(*[d._h for d in dsts])
+        B.check(self._lib.mmr_reshard_bind(self._h, sa, da, n))
+
     def SliceLocalShard(self, device: int, store: StoreHandle, wait: bool = True) -> int:
         p = C.c_void_p()
         fn = self._lib.mmr_store_shard_ptr if wait else self._lib.mmr_store_shard_ptr_async

@@ -169,7 +169,7 @@ int check_store(mmr_context* ctx, const mmr_store* s, const char* what) {
   return MMR_OK;
 }
 
-int reshard_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int n) {
+int reshard_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int n, bool launch = true) {
   if (n == 0) return MMR_OK;
   if (int rc = use_device(ctx)) return rc;
   std::vector<int64_t> ids;
@@ -191,13 +191,19 @@ int reshard_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* d
         return fail(MMR_INVALID_ARGUMENT, "store %lld is written by array %d and used again by array %d of the same batch",
                     (long long)dsts[a]->id, a, b);
 
-  ctx->stats.reshard_calls += 1;
+  if (launch) ctx->stats.reshard_calls += 1;
   Binding* binding = nullptr;
   auto bit = ctx->bindings.find(ids);
   if (bit != ctx->bindings.end()) {
     binding = bit->second.get();
-    ctx->stats.binding_cache_hits += 1;
+    if (launch) ctx->stats.binding_cache_hits += 1;
   } else {
+    // Building a plan or a pointer table allocates and copies: not allowed while the stream records a graph.
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(ctx->stream, &capture) == hipSuccess && capture != hipStreamCaptureStatusNone)
+      return fail(MMR_INVALID_ARGUMENT,
+                  "the stream is capturing and this reshard has no cached plan and pointer table yet: "
+                  "call mmr_reshard_bind (or run the reshard once) before the capture begins");
     std::vector<mmr_sharded_shape> sshapes(n), dshapes(n);
     for (int a = 0; a < n; ++a) {
       sshapes[a] = srcs[a]->shape;
@@ -220,6 +226,7 @@ int reshard_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* d
     binding = b.get();
     ctx->bindings.emplace(ids, std::move(b));
   }
+  if (!launch) return MMR_OK;
   const DevicePlan* dp = binding->plan;
   const mmr_plan& p = dp->plan;
   const uint32_t xm = p.options.xcd_mode;
@@ -560,6 +567,12 @@ int mmr_reshard_batch(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const
   if (!ctx || n < 0 || (n > 0 && (!srcs || !dsts))) return fail(MMR_INVALID_ARGUMENT, "bad batch arguments");
   std::lock_guard<std::mutex> lock(ctx->mu);
   return reshard_locked(ctx, srcs, dsts, n);
+}
+
+int mmr_reshard_bind(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int32_t n) {
+  if (!ctx || n < 0 || (n > 0 && (!srcs || !dsts))) return fail(MMR_INVALID_ARGUMENT, "bad batch arguments");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  return reshard_locked(ctx, srcs, dsts, n, /*launch=*/false);
 }
 
 int mmr_sync(mmr_context* ctx) {

@@ -384,3 +384,76 @@ def test_event_ordering_entry_points(ctx):
     mm._binding.check(lib.mmr_context_wait_event(ctx._h, ev))
     ctx.Sync()
     assert hip.hipEventDestroy(ev) == 0
+
+
+def test_reshard_replays_from_a_hip_graph():
+    """Once its plan and pointer table are bound, a reshard is kernel launches only.
+    Captured into a HIP graph, it is replayed three times with different data in the
+    stores, eager work and synchronisations of the same context in between; every
+    replay must match the oracle.  An unbound reshard during capture is refused
+    without breaking the capture."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so.7")  # the runtime the library already loaded
+    for fn in (hip.hipStreamBeginCapture, hip.hipStreamEndCapture, hip.hipGraphInstantiate, hip.hipGraphLaunch,
+               hip.hipGraphExecDestroy, hip.hipGraphDestroy):
+        fn.restype = C.c_int
+    hip.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+    hip.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+    hip.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_char_p, C.c_size_t]
+    hip.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+    hip.hipGraphExecDestroy.argtypes = [C.c_void_p]
+    hip.hipGraphDestroy.argtypes = [C.c_void_p]
+
+    ctx = mm.ReshardContext(0)  # a context of its own: a broken capture must not leak into other tests
+    try:
+        # mixed plan: aligned chunks (configuration 2 scaled), ragged rows (configuration 5 scaled), transposed layout
+        arrays = workloads.config(2, 8) + workloads.config(5, 16) + workloads.config(13, 16)
+        gs = [workloads.generate(a) for a in arrays]
+        srcs, dsts = make_stores(ctx, arrays, gs)
+        other = workloads.config(1, 16)
+        other_g = [workloads.generate(a) for a in other]
+        other_srcs, other_dsts = make_stores(ctx, other, other_g)
+
+        ctx.BindReshard(srcs, dsts)
+        ctx.Sync()
+        before = ctx.stats
+        stream = ctx.stream
+        say("capturing a batched reshard of %d arrays" % len(arrays))
+        assert hip.hipStreamBeginCapture(stream, 0) == 0  # hipStreamCaptureModeGlobal
+        with pytest.raises(mm.MmrError, match="capturing"):
+            ctx.Reshard(other_srcs[0], other_dsts[0])  # not bound: would allocate
+        ctx.ReshardBatch(srcs, dsts)
+        graph = C.c_void_p()
+        assert hip.hipStreamEndCapture(stream, C.byref(graph)) == 0
+        assert graph.value, "capture was invalidated"
+        assert ctx.stats["plans_built"] == before["plans_built"] and ctx.stats["bindings_built"] == before["bindings_built"]
+        exe = C.c_void_p()
+        assert hip.hipGraphInstantiate(C.byref(exe), graph, None, None, 0) == 0
+
+        rng = np.random.Generator(np.random.PCG64(99))
+        for replay in range(3):
+            if replay:  # new contents in the same source stores, junk in the destinations
+                for a, s, d in zip(arrays, srcs, dsts):
+                    g = rng.integers(0, 256, size=gs[arrays.index(a)].nbytes, dtype=np.uint8).view(
+                        gs[arrays.index(a)].dtype).reshape(gs[arrays.index(a)].shape)
+                    gs[arrays.index(a)] = g
+                    so = oracle_shape(a["type"], a["src"])
+                    shards = ro.make_shards(raw_global(a, g), so, a["src"].get("minor_to_major"))
+                    for dev in s.devices:
+                        ctx.AssembleShards(lib_shape(a["type"], a["src"]), dev, shards[dev].view(np.uint8).reshape(-1),
+                                           existing_store=s)
+                    junk = np.full(d.shard_bytes, 0xA5 + replay, dtype=np.uint8)
+                    for dev in d.devices:
+                        ctx.AssembleShards(lib_shape(a["type"], a["dst"]), dev, junk, existing_store=d)
+            say("graph replay %d" % replay)
+            assert hip.hipGraphLaunch(exe, stream) == 0
+            ctx.Sync()
+            _compare(arrays, gs, [read_all(ctx, d) for d in dsts])
+            # eager work of the same context between the replays
+            ctx.Reshard(other_srcs[0], other_dsts[0])
+            ctx.Sync()
+            _compare(other, other_g, [read_all(ctx, d) for d in other_dsts])
+        assert hip.hipGraphExecDestroy(exe) == 0
+        assert hip.hipGraphDestroy(graph) == 0
+    finally:
+        ctx.close()
