@@ -384,12 +384,31 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
   }
   const uint32_t order = options.order ? options.order : 2;
   if (order == 2 || order == 3) {
-    auto key = [order](const mmr_copy_chunk& c) {
-      return order == 2 ? std::make_pair(c.dst_slot, c.dst_off) : std::make_pair(c.src_slot, c.src_off);
+    // Sorting 72-byte records directly dominated the planning time of large batches: sort (key, index) triples
+    // and permute once.  The index as last key keeps equal keys (fill chunks share FILL as source) in emission order.
+    auto sort_copy = [order](std::vector<mmr_copy_chunk>& table) {
+      struct Key {
+        uint64_t slot, off;
+        uint32_t index;
+      };
+      std::vector<Key> keys(table.size());
+      bool sorted = true;
+      for (size_t i = 0; i < table.size(); ++i) {
+        const mmr_copy_chunk& c = table[i];
+        keys[i] = order == 2 ? Key{c.dst_slot, c.dst_off, static_cast<uint32_t>(i)}
+                             : Key{c.src_slot, c.src_off, static_cast<uint32_t>(i)};
+        if (i > 0 && std::tie(keys[i].slot, keys[i].off) < std::tie(keys[i - 1].slot, keys[i - 1].off)) sorted = false;
+      }
+      if (sorted) return;
+      std::sort(keys.begin(), keys.end(), [](const Key& a, const Key& b) {
+        return std::tie(a.slot, a.off, a.index) < std::tie(b.slot, b.off, b.index);
+      });
+      std::vector<mmr_copy_chunk> out(table.size());
+      for (size_t i = 0; i < keys.size(); ++i) out[i] = table[keys[i].index];
+      table.swap(out);
     };
-    auto cmp = [&](const mmr_copy_chunk& a, const mmr_copy_chunk& b) { return key(a) < key(b); };
-    std::stable_sort(plan->copy16.begin(), plan->copy16.end(), cmp);
-    std::stable_sort(plan->generic.begin(), plan->generic.end(), cmp);
+    sort_copy(plan->copy16);
+    sort_copy(plan->generic);
     // Tiles: by destination in blocks of 8 x 8 tiles rather than row after row, so the workgroups in flight
     // together cover a compact region with long contiguous pieces on the source side as well as on the
     // destination side (measured +10 % over plain destination order).
