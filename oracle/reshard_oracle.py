@@ -25,7 +25,7 @@ fills them (mm_sharding.cc:345-372, 427-431, 638-654):
     coordinate.
 
 Pinned by: brute force over single elements on tiny inputs
-(tests/test_oracle.py computes each element's owner tile by integer division,
+(tests/test_oracle_reshard.py computes each element's owner tile by integer division,
 independently of the slicing below), the round trip A->B->A, and the three
 device-order goldens of mm_sharding_test.cc:529-717 for the device <-> tile
 coordinate map.

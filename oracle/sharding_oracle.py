@@ -18,6 +18,12 @@ tests, re-expressed as numbers in tests/golden/sharding_golden.json:
   logical_to_physical_sharding
       src/pjrt_client/mm_sharding.cc:183-273
       pinned by mm_sharding_test.cc:101-228 (8 cases)
+  logical_sharding_to_op_sharding
+      src/pjrt_client/mpmd_logical_to_gspmd_sharding.cc:21-124
+      pinned by the OpShardings mpmd_logical_to_gspmd_sharding_test.cc:48-64,
+      190-205 expects (3 active cases, exact fields) and :116-187 (2 cases the
+      reference skips; given in XLA's canonical form, compared as tile dims
+      plus device order)
   canonicalize_sharding
       src/pjrt_client/mm_sharding.cc:275-456
       pinned by mm_sharding_test.cc:529-737 (3 golden descriptors, 1 error)

@@ -246,3 +246,37 @@ def test_logical_sharding_agrees_with_the_oracle(data):
         assert got["iota_transpose_perm"] == expect.iota_transpose_perm
         assert got["replicate_on_last_tile_dim"] == expect.replicate_on_last_tile_dim
         assert got["iota_offset"] == expect.iota_offset
+
+
+def test_logical_sharding_known_answers_of_the_reference():
+    """The OpShardings mpmd_logical_to_gspmd_sharding_test.cc expects, as numbers;
+    checked for the oracle restatement and for the C ABI.  Cases that carry a
+    `device_order` are given upstream in XLA's canonical HloSharding form: they are
+    compared as tile dims (without a trailing replication entry of size 1) plus
+    the order of devices over the tiles."""
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "sharding_golden.json")) as f:
+        cases = json.load(f)["logical_sharding_to_op_sharding"]
+    assert len(cases) >= 5
+    for c in cases:
+        pairs = [tuple(p) for p in c["logical_axes"]]
+        args = (c["mesh_dims"], c["mesh_axes"], pairs, c["names"], c["shape"], tuple(c["devices"]), c["total_devices"])
+        e = c["expect"]
+        o = so.logical_sharding_to_op_sharding(*args)
+        got_lib = mm.LogicalShardingToOpSharding(*args)
+        got = _op_dict(got_lib)
+        if "device_order" in e:
+            def strip(tile, repl):
+                return list(tile[:-1]) if repl and tile[-1] == 1 else list(tile)
+            assert strip(o.tile_assignment_dimensions, o.replicate_on_last_tile_dim) == e["tile_dims"], c["source"]
+            assert [int(d) for d in so.iota_tile_assignment(o).reshape(-1)] == e["device_order"], c["source"]
+            assert strip(got["tile_dims"], got["replicate_on_last_tile_dim"]) == e["tile_dims"], c["source"]
+            assert list(mm.TileAssignmentDevices(got_lib)) == e["device_order"], c["source"]
+            continue
+        assert (o.type, o.tile_assignment_dimensions, o.iota_reshape_dims, o.iota_transpose_perm, o.iota_offset,
+                o.replicate_on_last_tile_dim) == (e["type"], e["tile_dims"], e["iota_reshape_dims"],
+                                                  e["iota_transpose_perm"], e["iota_offset"],
+                                                  e["replicate_on_last_tile_dim"]), c["source"]
+        for k in e:
+            assert got[k] == e[k], (c["source"], k)
