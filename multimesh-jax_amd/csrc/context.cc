@@ -233,9 +233,9 @@ int reshard_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* d
   // aligned chunks: runs of 64 table neighbours per XCD measured best across the benchmark configurations
   MMR_HIP(mmr::launch_copy16(dp->d_copy16, static_cast<int64_t>(p.copy16.size()), binding->d_ptrs, xm == 0 ? 64 : xm,
                              ctx->stream));
-  // generic chunks leave partial lines at run boundaries; neighbours merge them when they share an L2.  Measured:
-  // small tables do best with one contiguous eighth per XCD, large ones with runs of 64 neighbours per XCD.
-  const uint32_t generic_xm = xm != 0 ? xm : (p.generic.size() <= 16384 ? 2u : 64u);
+  // generic chunks leave partial lines at run boundaries and share source lines with the chunks of neighbouring
+  // destination tiles; table neighbours merge both when they share an L2: runs of 64 per XCD (measured)
+  const uint32_t generic_xm = xm != 0 ? xm : 64u;
   MMR_HIP(mmr::launch_copy_generic(dp->d_generic, static_cast<int64_t>(p.generic.size()), binding->d_ptrs, generic_xm,
                                    ctx->stream));
   for (const DevicePlan::TransposeRun& run : dp->transpose_runs)

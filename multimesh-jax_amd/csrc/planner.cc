@@ -347,6 +347,11 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
     generic_chunk_bytes = static_cast<uint32_t>(std::min<int64_t>(std::max<int64_t>(payload / 16384, 4096), 8192)) & ~255u;
   }
   Builder builder(plan, chunk_bytes, generic_chunk_bytes, (options.flags & MMR_PLAN_ALL_GENERIC) != 0);
+  struct SlotInfo {
+    int array;
+    int64_t shard_bytes;
+  };
+  std::vector<SlotInfo> slot_info;  // by slot
   for (int a = 0; a < n; ++a) {
     Side S, D;
     if (int rc = make_side(srcs[a], &S)) return rc;
@@ -364,6 +369,8 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
     plan->srcs.push_back(srcs[a]);
     plan->dsts.push_back(dsts[a]);
     plan->slot_bases.push_back(plan->n_slots);
+    for (int64_t k = 0; k < S.dev_count; ++k) slot_info.push_back({a, S.shard_bytes});
+    for (int64_t k = 0; k < D.dev_count; ++k) slot_info.push_back({a, D.shard_bytes});
     if (int rc = plan_one_array(builder, S, D, static_cast<uint32_t>(plan->n_slots))) return rc;
     plan->n_slots += S.dev_count + D.dev_count;
   }
@@ -382,7 +389,10 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
       plan->copy16.clear();
     }
   }
+  // Default order: aligned chunks and transpose tiles by destination address; ragged (generic) chunks by
+  // destination with the tiles of an array interleaved (4), measured +12 % on configuration 5.
   const uint32_t order = options.order ? options.order : 2;
+  const uint32_t generic_order = options.order ? options.order : 4;
   if (order == 2 || order == 3) {
     // Sorting 72-byte records directly dominated the planning time of large batches: sort (key, index) triples
     // and permute once.  The index as last key keeps equal keys (fill chunks share FILL as source) in emission order.
@@ -408,7 +418,40 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
       table.swap(out);
     };
     sort_copy(plan->copy16);
-    sort_copy(plan->generic);
+    if (generic_order == order) sort_copy(plan->generic);
+  }
+  if (order == 4 || generic_order == 4) {
+    // Ragged rows: chunks of different destination tiles that cover the same rows read the same source lines at
+    // the edges of their column ranges.  Cut every destination buffer into equal fractions and keep the chunks of
+    // one fraction of all tiles of an array together (inside a fraction: by destination address), so that they
+    // run at the same time on the same XCD and the shared lines are fetched once.
+    const int64_t fraction_kib = (options.flags >> 8) & 0xffffu;  // tuning knob; 0 = default
+    const int64_t fraction_bytes = (fraction_kib ? fraction_kib : 64) * 1024;
+    auto sort_interleaved = [&](std::vector<mmr_copy_chunk>& table) {
+      struct Key {
+        uint64_t array, fraction, slot, off;
+        uint32_t index;
+      };
+      std::vector<Key> keys(table.size());
+      for (size_t i = 0; i < table.size(); ++i) {
+        const mmr_copy_chunk& c = table[i];
+        const SlotInfo& info = slot_info[c.dst_slot];
+        const uint64_t fractions = std::max<int64_t>(1, info.shard_bytes / fraction_bytes);
+        keys[i] = Key{static_cast<uint64_t>(info.array),
+                      info.shard_bytes > 0 ? c.dst_off * fractions / static_cast<uint64_t>(info.shard_bytes) : 0, c.dst_slot,
+                      c.dst_off, static_cast<uint32_t>(i)};
+      }
+      std::sort(keys.begin(), keys.end(), [](const Key& a, const Key& b) {
+        return std::tie(a.array, a.fraction, a.slot, a.off, a.index) < std::tie(b.array, b.fraction, b.slot, b.off, b.index);
+      });
+      std::vector<mmr_copy_chunk> out(table.size());
+      for (size_t i = 0; i < keys.size(); ++i) out[i] = table[keys[i].index];
+      table.swap(out);
+    };
+    if (order == 4) sort_interleaved(plan->copy16);
+    sort_interleaved(plan->generic);
+  }
+  if (order == 2 || order == 3 || order == 4) {
     // Tiles: by destination in blocks of 8 x 8 tiles rather than row after row, so the workgroups in flight
     // together cover a compact region with long contiguous pieces on the source side as well as on the
     // destination side (measured +10 % over plain destination order).
@@ -421,7 +464,7 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
     };
     std::stable_sort(plan->transposes.begin(), plan->transposes.end(),
                      [&](const mmr_transpose_chunk& a, const mmr_transpose_chunk& b) {
-                       return order == 2 ? tile_key(a) < tile_key(b)
+                       return order != 3 ? tile_key(a) < tile_key(b)
                                          : std::make_pair(a.src_slot, a.src_off) < std::make_pair(b.src_slot, b.src_off);
                      });
   }

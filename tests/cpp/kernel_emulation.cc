@@ -153,7 +153,7 @@ int mmr_emulate_plan(const mmr_plan* plan, void* const* slot_ptrs, const size_t*
     const int64_t n = mmr_plan_get_copy_chunks(plan, kind, nullptr, 0);
     std::vector<mmr_copy_chunk> chunks(static_cast<size_t>(n));
     mmr_plan_get_copy_chunks(plan, kind, chunks.data(), n);
-    const uint32_t mode = kind == 0 ? (xcd_mode == 0 ? 64 : xcd_mode) : (xcd_mode == 0 ? 2 : xcd_mode);
+    const uint32_t mode = kind == 0 ? (xcd_mode == 0 ? 64 : xcd_mode) : (xcd_mode == 0 ? 64 : xcd_mode);
     for_each_chunk(n, mode, [&](uint32_t ci) {
       const mmr_copy_chunk& c = chunks[ci];
       if (c.dst_slot >= n_slots || (c.src_slot != MMR_SLOT_FILL && c.src_slot >= n_slots)) {
