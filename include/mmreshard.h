@@ -183,6 +183,7 @@ typedef struct {
 } mmr_transpose_chunk;
 
 #define MMR_PLAN_ALL_GENERIC 1u
+#define MMR_PLAN_NO_AUTOTUNE 2u
 
 typedef struct {
   uint32_t chunk_bytes; /* target bytes per copy chunk, 0 = default */
@@ -193,6 +194,8 @@ typedef struct {
                            consecutive workgroups round-robin over the 8 XCDs); 2 = each XCD takes a contiguous
                            eighth of the table; G >= 16 = runs of G table neighbours share an XCD (and its L2) */
   uint32_t flags;       /* MMR_PLAN_ALL_GENERIC: route aligned chunks through the generic kernel too (testing);
+                           MMR_PLAN_NO_AUTOTUNE: keep the default table order instead of timing a few orders on
+                           the first reshard of a descriptor pair (only done when `order` is 0);
                            bits 8-23: KiB per tile and fraction for order 4 (0 = default, 64) */
 } mmr_plan_options;
 
@@ -207,6 +210,9 @@ typedef struct {
   int64_t bytes_filled;        /* pad bytes zeroed */
   int64_t table_bytes;         /* device-resident plan size */
   int64_t n_slots;
+  int64_t order_used;          /* table order in effect: 0 = the default mix, else a value of mmr_plan_options.order */
+  int64_t interleave_kib;      /* order 4 only: KiB per tile and fraction */
+  int64_t orders_timed;        /* how many table orders the first reshard timed (0 = no tuning) */
 } mmr_plan_stats;
 
 int mmr_plan_create(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int32_t n_arrays,

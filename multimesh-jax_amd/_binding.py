@@ -80,7 +80,8 @@ class PlanOptions(C.Structure):
 class PlanStats(C.Structure):
     _fields_ = [(n, C.c_int64) for n in (
         "n_arrays", "n_boxes", "n_copy16_chunks", "n_copy_generic_chunks", "n_transpose_chunks",
-        "n_fill_chunks", "bytes_moved", "bytes_filled", "table_bytes", "n_slots")]
+        "n_fill_chunks", "bytes_moved", "bytes_filled", "table_bytes", "n_slots", "order_used", "interleave_kib",
+        "orders_timed")]
 
     def as_dict(self):
         return {n: getattr(self, n) for n, _ in self._fields_}

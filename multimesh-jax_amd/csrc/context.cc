@@ -40,6 +40,7 @@ struct DevicePlan {
     int64_t begin, count;
   };
   std::vector<TransposeRun> transpose_runs;  // the table is sorted by itemsize; one launch per run
+  bool tuned = false;                        // the table order has been chosen (timed or fixed by the options)
 };
 
 struct Binding {
@@ -129,21 +130,19 @@ void drop_bindings_of(mmr_context* ctx, int64_t store_id) {
   }
 }
 
-int get_plan(mmr_context* ctx, const std::vector<mmr_sharded_shape>& srcs, const std::vector<mmr_sharded_shape>& dsts,
-             DevicePlan** out) {
+void free_tables(DevicePlan* dp) {
+  (void)hipFree(dp->d_copy16);
+  (void)hipFree(dp->d_generic);
+  (void)hipFree(dp->d_transposes);
+  dp->d_copy16 = dp->d_generic = nullptr;
+  dp->d_transposes = nullptr;
+}
+
+// Plans n descriptor pairs under `options` and uploads the tables (not cached here).
+int make_device_plan(mmr_context* ctx, const std::vector<mmr_sharded_shape>& srcs, const std::vector<mmr_sharded_shape>& dsts,
+                     const mmr_plan_options& options, DevicePlan* dp) {
   const int n = static_cast<int>(srcs.size());
-  std::string key = mmr::plan_key(srcs.data(), dsts.data(), n, ctx->options);
-  auto it = ctx->plans.find(key);
-  if (it != ctx->plans.end()) {
-    ctx->stats.plan_cache_hits += 1;
-    *out = it->second.get();
-    return MMR_OK;
-  }
-  auto dp = std::make_unique<DevicePlan>();
-  if (int rc = mmr::build_plan(srcs.data(), dsts.data(), n, ctx->options, &dp->plan)) return rc;
-  if (int rc = upload(ctx, dp->plan.copy16, &dp->d_copy16)) return rc;
-  if (int rc = upload(ctx, dp->plan.generic, &dp->d_generic)) return rc;
-  if (int rc = upload(ctx, dp->plan.transposes, &dp->d_transposes)) return rc;
+  if (int rc = mmr::build_plan(srcs.data(), dsts.data(), n, options, &dp->plan)) return rc;
   const std::vector<mmr_transpose_chunk>& tr = dp->plan.transposes;
   for (const mmr_transpose_chunk& c : tr) {  // the kernel's LDS tile and lane mapping assume these bounds
     uint32_t tile_x = 0, tile_y = 0;
@@ -157,10 +156,123 @@ int get_plan(mmr_context* ctx, const std::vector<mmr_sharded_shape>& srcs, const
     if (i == 0 || tr[i].itemsize != tr[i - 1].itemsize) dp->transpose_runs.push_back({tr[i].itemsize, i, 0});
     dp->transpose_runs.back().count += 1;
   }
+  if (int rc = upload(ctx, dp->plan.copy16, &dp->d_copy16)) return rc;
+  if (int rc = upload(ctx, dp->plan.generic, &dp->d_generic)) return rc;
+  if (int rc = upload(ctx, dp->plan.transposes, &dp->d_transposes)) return rc;
+  return MMR_OK;
+}
+
+int get_plan(mmr_context* ctx, const std::vector<mmr_sharded_shape>& srcs, const std::vector<mmr_sharded_shape>& dsts,
+             DevicePlan** out) {
+  const int n = static_cast<int>(srcs.size());
+  std::string key = mmr::plan_key(srcs.data(), dsts.data(), n, ctx->options);
+  auto it = ctx->plans.find(key);
+  if (it != ctx->plans.end()) {
+    ctx->stats.plan_cache_hits += 1;
+    *out = it->second.get();
+    return MMR_OK;
+  }
+  auto dp = std::make_unique<DevicePlan>();
+  if (int rc = make_device_plan(ctx, srcs, dsts, ctx->options, dp.get())) {
+    free_tables(dp.get());
+    return rc;
+  }
   ctx->stats.plans_built += 1;
   *out = dp.get();
   ctx->plans.emplace(std::move(key), std::move(dp));
   return MMR_OK;
+}
+
+// One launch per kernel class over the plan's tables.
+int launch_plan(mmr_context* ctx, const DevicePlan* dp, void* const* d_ptrs) {
+  const mmr_plan& p = dp->plan;
+  const uint32_t xm = p.options.xcd_mode;
+  // aligned chunks: runs of 64 table neighbours per XCD measured best across the benchmark configurations
+  MMR_HIP(mmr::launch_copy16(dp->d_copy16, static_cast<int64_t>(p.copy16.size()), d_ptrs, xm == 0 ? 64 : xm, ctx->stream));
+  // generic chunks leave partial lines at run boundaries and share source lines with the chunks of neighbouring
+  // destination tiles; table neighbours merge both when they share an L2: runs of 64 per XCD (measured)
+  MMR_HIP(mmr::launch_copy_generic(dp->d_generic, static_cast<int64_t>(p.generic.size()), d_ptrs, xm == 0 ? 64 : xm,
+                                   ctx->stream));
+  for (const DevicePlan::TransposeRun& run : dp->transpose_runs)
+    // tiles are ordered in 8 x 8 blocks; runs of 64 table neighbours per XCD keep a block in one L2 (measured best)
+    MMR_HIP(mmr::launch_transpose(dp->d_transposes + run.begin, run.count, d_ptrs, xm == 0 ? 64 : xm, run.itemsize,
+                                  ctx->stream));
+  return MMR_OK;
+}
+
+int64_t launches_of(const DevicePlan* dp) {
+  return (dp->plan.copy16.empty() ? 0 : 1) + (dp->plan.generic.empty() ? 0 : 1) +
+         static_cast<int64_t>(dp->transpose_runs.size());
+}
+
+// Which order of the chunk tables is fastest depends on how the two tilings interleave in memory (measured: plain
+// destination order for configurations 1, 2 and 4, destination tiles interleaved in 4 MiB fractions for
+// configuration 3, in 64 KiB fractions for ragged rows).  The first reshard of a descriptor pair therefore times a
+// few orders on the caller's own buffers (a reshard is idempotent) and keeps the fastest; the choice is cached with
+// the plan.  Blocks the calling thread for those few launches.
+int tune_plan(mmr_context* ctx, DevicePlan* dp, void* const* d_ptrs) {
+  dp->tuned = true;
+  const mmr_plan_options base = dp->plan.options;
+  const size_t chunks = dp->plan.copy16.size() + dp->plan.generic.size();
+  if (base.order != 0 || (base.flags & MMR_PLAN_NO_AUTOTUNE) || chunks < 1024 || chunks > 262144) return MMR_OK;
+  struct Candidate {
+    uint32_t order, kib;
+  };
+  const Candidate candidates[] = {{4, 64}, {4, 1024}, {4, 4096}, {2, 0}};
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  MMR_HIP(hipEventCreate(&e0));
+  MMR_HIP(hipEventCreate(&e1));
+  auto time_plan = [&](const DevicePlan* plan, float* ms) -> int {
+    if (int rc = launch_plan(ctx, plan, d_ptrs)) return rc;  // warm-up
+    MMR_HIP(hipEventRecord(e0, ctx->stream));
+    for (int i = 0; i < 3; ++i)
+      if (int rc = launch_plan(ctx, plan, d_ptrs)) return rc;
+    MMR_HIP(hipEventRecord(e1, ctx->stream));
+    MMR_HIP(hipEventSynchronize(e1));
+    MMR_HIP(hipEventElapsedTime(ms, e0, e1));
+    return MMR_OK;
+  };
+  int rc = MMR_OK;
+  float best_ms = 0;
+  int64_t timed = 1;
+  rc = time_plan(dp, &best_ms);
+  std::unique_ptr<DevicePlan> best;
+  for (const Candidate& cand : candidates) {
+    if (rc != MMR_OK) break;
+    if (cand.order == 2 && dp->plan.generic.empty()) continue;  // the default already is order 2 for aligned chunks
+    if (cand.order == 4 && cand.kib == 64 && dp->plan.copy16.empty()) continue;  // ... and 4 / 64 KiB for ragged ones
+    mmr_plan_options o = base;
+    o.order = cand.order;
+    o.flags = (o.flags & 0xffu) | (cand.kib << 8);
+    auto alt = std::make_unique<DevicePlan>();
+    rc = make_device_plan(ctx, dp->plan.srcs, dp->plan.dsts, o, alt.get());
+    float ms = 0;
+    if (rc == MMR_OK) rc = time_plan(alt.get(), &ms);
+    if (rc == MMR_OK) timed += 1;
+    if (rc == MMR_OK && ms < 0.98f * best_ms) {  // only a clear win replaces the default
+      best_ms = ms;
+      if (best) free_tables(best.get());
+      best = std::move(alt);
+    } else {
+      (void)hipStreamSynchronize(ctx->stream);
+      free_tables(alt.get());
+    }
+  }
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  if (rc == MMR_OK && best) {  // the cached object keeps its address: bindings point at it
+    free_tables(dp);
+    dp->plan = std::move(best->plan);
+    dp->d_copy16 = best->d_copy16;
+    dp->d_generic = best->d_generic;
+    dp->d_transposes = best->d_transposes;
+    dp->transpose_runs = std::move(best->transpose_runs);
+    dp->plan.options = base;  // still the plan of the context's options
+  } else if (best) {
+    free_tables(best.get());
+  }
+  dp->plan.stats.orders_timed = timed;
+  return rc;
 }
 
 int check_store(mmr_context* ctx, const mmr_store* s, const char* what) {
@@ -227,23 +339,19 @@ int reshard_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* d
     ctx->bindings.emplace(ids, std::move(b));
   }
   if (!launch) return MMR_OK;
-  const DevicePlan* dp = binding->plan;
-  const mmr_plan& p = dp->plan;
-  const uint32_t xm = p.options.xcd_mode;
-  // aligned chunks: runs of 64 table neighbours per XCD measured best across the benchmark configurations
-  MMR_HIP(mmr::launch_copy16(dp->d_copy16, static_cast<int64_t>(p.copy16.size()), binding->d_ptrs, xm == 0 ? 64 : xm,
-                             ctx->stream));
-  // generic chunks leave partial lines at run boundaries and share source lines with the chunks of neighbouring
-  // destination tiles; table neighbours merge both when they share an L2: runs of 64 per XCD (measured)
-  const uint32_t generic_xm = xm != 0 ? xm : 64u;
-  MMR_HIP(mmr::launch_copy_generic(dp->d_generic, static_cast<int64_t>(p.generic.size()), binding->d_ptrs, generic_xm,
-                                   ctx->stream));
-  for (const DevicePlan::TransposeRun& run : dp->transpose_runs)
-    // tiles are ordered in 8 x 8 blocks; runs of 64 table neighbours per XCD keep a block in one L2 (measured best)
-    MMR_HIP(mmr::launch_transpose(dp->d_transposes + run.begin, run.count, binding->d_ptrs, xm == 0 ? 64 : xm, run.itemsize,
-                                  ctx->stream));
-  ctx->stats.kernel_launches +=
-      (p.copy16.empty() ? 0 : 1) + (p.generic.empty() ? 0 : 1) + static_cast<int64_t>(dp->transpose_runs.size());
+  DevicePlan* dp = binding->plan;
+  if (!dp->tuned) {
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(ctx->stream, &capture) == hipSuccess && capture != hipStreamCaptureStatusNone) {
+      // recorded into a graph as it is: the graph keeps the addresses of these tables, so they must never be
+      // replaced by a later tuning run
+      dp->tuned = true;
+    } else if (int rc = tune_plan(ctx, dp, binding->d_ptrs)) {
+      return rc;
+    }
+  }
+  if (int rc = launch_plan(ctx, dp, binding->d_ptrs)) return rc;
+  ctx->stats.kernel_launches += launches_of(dp);
   return MMR_OK;
 }
 

@@ -472,6 +472,8 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
   // itemsize, the order above kept inside each run
   std::stable_sort(plan->transposes.begin(), plan->transposes.end(),
                    [](const mmr_transpose_chunk& a, const mmr_transpose_chunk& b) { return a.itemsize < b.itemsize; });
+  plan->stats.order_used = options.order;
+  plan->stats.interleave_kib = options.order == 4 ? (((options.flags >> 8) & 0xffffu) ? ((options.flags >> 8) & 0xffffu) : 64) : 0;
   plan->stats.n_arrays = n;
   plan->stats.n_copy16_chunks = static_cast<int64_t>(plan->copy16.size());
   plan->stats.n_copy_generic_chunks = static_cast<int64_t>(plan->generic.size());

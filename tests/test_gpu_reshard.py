@@ -457,3 +457,29 @@ def test_reshard_replays_from_a_hip_graph():
         assert hip.hipGraphDestroy(graph) == 0
     finally:
         ctx.close()
+
+
+def test_table_order_is_tuned_on_first_use_and_results_do_not_change():
+    """The first reshard of a descriptor pair times a few table orders on the caller's
+    buffers and keeps the fastest; whichever wins, the bytes are the oracle's.  A fixed
+    order or MMR_PLAN_NO_AUTOTUNE switches the tuning off."""
+    arrays = workloads.config(3, 2)  # 4,096 aligned chunks
+    gs = [workloads.generate(a) for a in arrays]
+    for flags, order, tuned in ((0, 0, True), (2, 0, False), (0, 2, False)):
+        ctx = mm.ReshardContext(0)
+        try:
+            ctx.set_plan_options(0, order, 0, flags)
+            outs, srcs, dsts = gpu_reshard(ctx, arrays, gs, keep=True)
+            _compare(arrays, gs, outs)
+            st = ctx.plan_stats(srcs[0], dsts[0])
+            say("flags %d order %d: %d orders timed, order used %d / %d KiB" % (
+                flags, order, st["orders_timed"], st["order_used"], st["interleave_kib"]))
+            assert (st["orders_timed"] >= 2) == tuned
+            # a second reshard of the same stores reuses the tuned plan: no further timing, same bytes
+            before = ctx.stats["kernel_launches"]
+            ctx.Reshard(srcs[0], dsts[0])
+            ctx.Sync()
+            assert ctx.stats["kernel_launches"] - before == 1
+            _compare(arrays, gs, [read_all(ctx, d) for d in dsts])
+        finally:
+            ctx.close()
