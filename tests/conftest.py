@@ -17,7 +17,8 @@ def pytest_configure(config):
     if not os.path.exists(os.path.join(ROOT, "oracle", "libreshard_oracle.so")):
         subprocess.check_call(["make", "-s", "-C", os.path.join(ROOT, "oracle")])
     if not (os.path.exists(os.path.join(ROOT, "tests", "cpp", "libmmr_emulation.so"))
-            and os.path.exists(os.path.join(ROOT, "tests", "cpp", "hip_execute_context_test"))):
+            and os.path.exists(os.path.join(ROOT, "tests", "cpp", "hip_execute_context_test"))
+            and os.path.exists(os.path.join(ROOT, "tests", "cpp", "sanitize_sweep"))):
         subprocess.check_call(["bash", os.path.join(ROOT, "tests", "cpp", "build.sh")])
 
 

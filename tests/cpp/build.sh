@@ -15,3 +15,10 @@ g++ -O2 -std=c++17 -Wall -Wextra -Wno-unknown-pragmas -fPIC -shared -I"${root}/i
   -Wl,-rpath,'$ORIGIN/../../multimesh-jax_amd' -Wl,-rpath,/opt/rocm/lib \
   -o "${here}/libmmr_emulation.so"
 echo "built ${here}/libmmr_emulation.so"
+# Host-only sanitizer build: planner + descriptor geometry + the emulation of the kernels + a random sweep.
+g++ -O1 -g -std=c++17 -fsanitize=address,undefined -fno-sanitize-recover=undefined -fno-omit-frame-pointer \
+  -Wall -Wextra -Wno-unknown-pragmas -I"${root}/include" -I"${root}/multimesh-jax_amd/csrc" \
+  "${root}/multimesh-jax_amd/csrc/geometry.cc" "${root}/multimesh-jax_amd/csrc/sharding_frontend.cc" \
+  "${root}/multimesh-jax_amd/csrc/planner.cc" "${here}/kernel_emulation.cc" "${here}/sanitize_sweep.cc" \
+  -o "${here}/sanitize_sweep"
+echo "built ${here}/sanitize_sweep"

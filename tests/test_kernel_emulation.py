@@ -115,3 +115,18 @@ def test_transposed_benchmark_workloads_scaled():
         arrays = workloads.config(index, 16)
         gs = [workloads.generate(a) for a in arrays]
         _check(arrays, gs)
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_sanitizer_sweep_of_planner_and_kernel_code(seed):
+    """tests/cpp/sanitize_sweep: planner, descriptor geometry and the kernels' per-chunk code built with the address
+    and undefined-behaviour sanitizers (host only), 1,500 random sharding pairs checked element by element."""
+    import os
+    import subprocess
+    here = os.path.dirname(os.path.abspath(__file__))
+    exe = os.path.join(here, "cpp", "sanitize_sweep")
+    if not os.path.exists(exe):
+        subprocess.check_call(["bash", os.path.join(here, "cpp", "build.sh")])
+    p = subprocess.run([exe, "1500", str(seed)], capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stdout + p.stderr
+    assert "cases OK" in p.stdout
