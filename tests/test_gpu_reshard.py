@@ -483,3 +483,36 @@ def test_table_order_is_tuned_on_first_use_and_results_do_not_change():
             _compare(arrays, gs, [read_all(ctx, d) for d in dsts])
         finally:
             ctx.close()
+
+
+def test_concurrent_callers(ctx):
+    """Several host threads resharding at once: four on one shared context (calls serialise on the context's
+    lock, work on its one stream) and two with a context each (two streams on the GPU at the same time).
+    ctypes drops the GIL during the calls, so they really overlap."""
+    import threading
+
+    def job(context, index, errors):
+        try:
+            arrays = workloads.config((1, 5, 13, 3)[index % 4], 8)
+            gs = [workloads.generate(a) for a in arrays]
+            for _ in range(3):
+                outs = gpu_reshard(context, arrays, gs)
+                _compare(arrays, gs, outs)
+        except BaseException as e:  # noqa: BLE001 - reported by the main thread
+            errors.append((index, repr(e)))
+
+    errors = []
+    own = [mm.ReshardContext(0), mm.ReshardContext(0)]
+    try:
+        threads = [threading.Thread(target=job, args=(ctx, i, errors)) for i in range(4)]
+        threads += [threading.Thread(target=job, args=(own[i], 4 + i, errors)) for i in range(2)]
+        say("six threads, three contexts")
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join(timeout=100)
+            assert not t.is_alive(), "a resharding thread did not finish"
+        assert not errors, errors
+    finally:
+        for c in own:
+            c.close()
