@@ -9,6 +9,8 @@
 
 namespace mmr {
 
+// Flat device-to-device copy; both pointers and the size must be multiples of 16 (hipErrorInvalidValue otherwise).
+hipError_t launch_flat_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);
 // Chunks whose offsets, strides and widths are all multiples of 16 bytes.
 // xcd_mode: 0/1 = chunk i runs as workgroup i (the hardware deals consecutive
 // workgroups round-robin over the 8 XCDs); 2 = each XCD takes a contiguous

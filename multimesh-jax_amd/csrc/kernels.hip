@@ -156,6 +156,31 @@ __global__ __launch_bounds__(TransposeTile<sizeof(T)>::kThreads) void mmr_transp
   transpose_tiles<T>(c, src, dst, lds);
 }
 
+// Flat copy of `vectors` 16-byte vectors: workgroup i moves the i-th block of kFlatVectors vectors, all loads of a
+// lane before its first store.  AssembleShards of a device-resident shard (one flat copy of the shard's bytes).
+constexpr uint32_t kFlatVectors = 512;  // 8 KiB per workgroup, like the plan's chunks
+
+__global__ __launch_bounds__(256) void mmr_flat_copy_kernel(const void* __restrict__ src_, void* __restrict__ dst_,
+                                                            uint64_t vectors) {
+  typedef DeviceMem<true, true> M;
+  const uint64_t base = static_cast<uint64_t>(blockIdx.x) * kFlatVectors;
+  gcchar* src = (gcchar*)(static_cast<const char*>(src_)) + (base << 4);
+  gchar* dst = (gchar*)(static_cast<char*>(dst_)) + (base << 4);
+  const uint64_t left = vectors - base;
+  const uint32_t n = left < kFlatVectors ? static_cast<uint32_t>(left) : kFlatVectors;
+  V16 v[kFlatVectors / 256];
+#pragma unroll
+  for (uint32_t u = 0; u < kFlatVectors / 256; ++u) {
+    const uint32_t i = threadIdx.x + u * 256;
+    if (i < n) v[u] = M::load16(src + (static_cast<int64_t>(i) << 4));
+  }
+#pragma unroll
+  for (uint32_t u = 0; u < kFlatVectors / 256; ++u) {
+    const uint32_t i = threadIdx.x + u * 256;
+    if (i < n) M::store16(dst + (static_cast<int64_t>(i) << 4), v[u]);
+  }
+}
+
 hipError_t check_grid(int64_t n) { return (n < 0 || n > 0x7ff00000LL) ? hipErrorInvalidValue : hipSuccess; }
 
 }  // namespace
@@ -163,6 +188,16 @@ hipError_t check_grid(int64_t n) { return (n < 0 || n > 0x7ff00000LL) ? hipError
 // Launch shapes are the measured optimum on MI355X for 8 KiB (aligned) and
 // 4 KiB (generic) chunks: 256 threads, up to 8 (aligned) or 2 (generic) 16-byte
 // accesses in flight per lane before the first store.
+hipError_t launch_flat_copy(const void* src, void* dst, size_t bytes, hipStream_t stream) {
+  if (bytes == 0) return hipSuccess;
+  if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst) | bytes) & 15u) return hipErrorInvalidValue;
+  const uint64_t vectors = bytes >> 4;
+  const uint64_t blocks = (vectors + kFlatVectors - 1) / kFlatVectors;
+  if (hipError_t e = check_grid(static_cast<int64_t>(blocks))) return e;
+  hipLaunchKernelGGL(mmr_flat_copy_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, stream, src, dst, vectors);
+  return hipGetLastError();
+}
+
 hipError_t launch_copy16(const mmr_copy_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
                          hipStream_t stream) {
   if (n == 0) return hipSuccess;

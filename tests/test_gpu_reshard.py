@@ -516,3 +516,36 @@ def test_concurrent_callers(ctx):
     finally:
         for c in own:
             c.close()
+
+
+def test_device_resident_shards_assemble_through_the_copy_kernel(ctx):
+    """AssembleShards of a large device-resident shard (the GPU branch of AssembleShardsImpl,
+    zuku_execute_context_impl.cc:405-415) runs the library's flat copy kernel; sizes that are not a multiple of 16
+    finish through the runtime.  Bytes must arrive unchanged, bytes beyond `size` must stay untouched."""
+    n = 48 * 1024 * 1024 + 16  # bytes per shard
+    shape = mm.sharded_shape("U8", [(2 * n, 2, 0)], 0, 2)
+    rng = np.random.Generator(np.random.PCG64(5))
+    data = rng.integers(0, 256, size=n, dtype=np.uint8)
+    src = ctx.CreateStore(shape, name="assemble.src")
+    ctx.AssembleShards(shape, 0, data, existing_store=src)
+    ptr = ctx.SliceLocalShard(0, src)
+    dst = ctx.CreateStore(shape, name="assemble.dst")
+    for size in (n, n - 5, (1 << 20) + 16, 4096):
+        ctx.AssembleShards(shape, 1, np.full(n, 0x77, dtype=np.uint8), existing_store=dst)
+        before = ctx.stats["kernel_launches"]
+        ctx.AssembleShards(shape, 1, ptr, existing_store=dst, size=size)
+        ctx.Sync()
+        assert ctx.stats["kernel_launches"] - before == (1 if size >= (1 << 20) else 0)
+        got = ctx.ReadShard(dst, 1)
+        assert got[:size].tobytes() == data[:size].tobytes(), size
+        assert (got[size:] == 0x77).all(), size
+    # rate of the device-to-device assemble
+    reps = 20
+    ctx.Sync()
+    ctx.StartTimer()
+    for _ in range(reps):
+        ctx.AssembleShards(shape, 1, ptr, existing_store=dst, size=n)
+    ms = ctx.StopTimer() / reps
+    say("device-to-device AssembleShards of %d MiB: %.1f us, %.0f GB/s (read + write)" % (n >> 20, ms * 1e3, 2 * n / ms / 1e6))
+    for s in (src, dst):
+        ctx.Free(s)
