@@ -109,6 +109,9 @@ def config(index: int, scale: int = 1) -> List[dict]:
         shape = (8192 // s, 8192 // s)
         return [_array("transposed", type_, shape, _side(shape, (4, 1), 0),
                        _side(shape, (1, 4), 4, minor_to_major=(0, 1)), 13, "raw")]
+    if index == 16:  # probe: configuration 10's split with 16-byte aligned pieces (816 / 544 / 272-byte rows)
+        b = (88064 // s, 4080)
+        return [_array("probe_u8_aligned", "U8", b, _side(b, (1, 3), 0), _side(b, (1, 5), 3), 6, "raw")]
     if index == 7:  # probe: 4-byte elements, uneven 3-way -> 5-way (dword-aligned, not 16-byte-aligned runs)
         b = (11008 // s, 1025)
         return [_array("probe_s32", "S32", b, _side(b, (1, 3), 0), _side(b, (1, 5), 3), 7, "raw")]
