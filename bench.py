@@ -78,6 +78,9 @@ def measure(ctx, mm, workloads, args, config, with_parity=True):
         srcs, dsts = sets[i % len(sets)]
         if len(srcs) == 1:
             ctx.Reshard(srcs[0], dsts[0])
+        elif args.unbatched:  # one call and one launch per array, as the reference's schedule loop issues them
+            for s_, d_ in zip(srcs, dsts):
+                ctx.Reshard(s_, d_)
         else:
             ctx.ReshardBatch(srcs, dsts)
 
@@ -148,6 +151,8 @@ def main():
     ap.add_argument("--sets", type=int, default=3, help="independent buffer sets rotated between steps")
     ap.add_argument("--all", action="store_true", help="also measure configurations 1, 3, 4 and 5 (adds minutes)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--unbatched", action="store_true",
+                    help="multi-array configurations: one Reshard call per array instead of one batched call (probing)")
     # plan options (0 = library default) and probing switches
     ap.add_argument("--chunk-bytes", type=int, default=0)
     ap.add_argument("--order", type=int, default=0)

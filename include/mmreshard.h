@@ -312,6 +312,10 @@ int mmr_reshard_batch(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const
  * fails with MMR_INVALID_ARGUMENT and leaves the capture intact).  Schedule-build
  * time work like MpmdScheduler::AddReshardTask, mpmd_partition.cc:340-351. */
 int mmr_reshard_bind(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int32_t n);
+/* The argument checks of mmr_reshard without planning or launching anything (both stores of this context, distinct,
+ * resident, same type and global extents): lets a caller that queues Reshard calls of one schedule window
+ * (mm_pjrt_executable.cc:616-658) for a single mmr_reshard_batch report a bad call where it is made. */
+int mmr_reshard_validate(mmr_context* ctx, mmr_store* src, mmr_store* dst);
 
 /* Build and upload the plan of n descriptor pairs (one batch) ahead of the first
  * reshard, i.e. when the schedule entry is created (MpmdScheduler::AddReshardTask,

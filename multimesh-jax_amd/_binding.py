@@ -150,6 +150,7 @@ PROTOTYPES = {
     "mmr_reshard": (C.c_int, [VP, VP, VP]),
     "mmr_reshard_batch": (C.c_int, [VP, P(VP), P(VP), I32]),
     "mmr_reshard_bind": (C.c_int, [VP, P(VP), P(VP), I32]),
+    "mmr_reshard_validate": (C.c_int, [VP, VP, VP]),
     "mmr_sync": (C.c_int, [VP]),
     "mmr_timer_start": (C.c_int, [VP]),
     "mmr_timer_stop": (C.c_int, [VP, P(C.c_float)]),

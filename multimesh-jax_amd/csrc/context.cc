@@ -689,6 +689,27 @@ int mmr_reshard_batch(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const
   return reshard_locked(ctx, srcs, dsts, n);
 }
 
+int mmr_reshard_validate(mmr_context* ctx, mmr_store* src, mmr_store* dst) {
+  if (!ctx) return fail(MMR_INVALID_ARGUMENT, "null context");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  if (int rc = check_store(ctx, src, "source")) return rc;
+  if (int rc = check_store(ctx, dst, "destination")) return rc;
+  if (src == dst) return fail(MMR_INVALID_ARGUMENT, "source and destination are the same store");
+  if (src->offloaded() || dst->offloaded())
+    return fail(MMR_INVALID_ARGUMENT, "store %lld is still offloaded to host memory",
+                (long long)(src->offloaded() ? src->id : dst->id));
+  const mmr::Side& S = src->side;
+  const mmr::Side& D = dst->side;
+  if (S.dtype != D.dtype)
+    return fail(MMR_INVALID_ARGUMENT, "source type %d differs from destination type %d", S.dtype, D.dtype);
+  if (S.rank != D.rank) return fail(MMR_INVALID_ARGUMENT, "source rank %d differs from destination rank %d", S.rank, D.rank);
+  for (int i = 0; i < S.rank; ++i)
+    if (S.size[i] != D.size[i])
+      return fail(MMR_INVALID_ARGUMENT, "dim %d is %lld in the source and %lld in the destination", i,
+                  (long long)S.size[i], (long long)D.size[i]);
+  return MMR_OK;
+}
+
 int mmr_reshard_bind(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int32_t n) {
   if (!ctx || n < 0 || (n > 0 && (!srcs || !dsts))) return fail(MMR_INVALID_ARGUMENT, "bad batch arguments");
   std::lock_guard<std::mutex> lock(ctx->mu);

@@ -87,6 +87,7 @@ std::shared_ptr<HipExecuteContext> HipExecuteContext::Create(std::set<int> local
 }
 
 HipExecuteContext::~HipExecuteContext() {
+  pending_.clear();    // work nobody waited for
   in_flight_.clear();  // drops the stores still attached to half-arrived ops
   // Handles may outlive the context (Python shutdown order in the reference,
   // zuku_execute_context_impl.cc:64-71); their stores die with the context.
@@ -151,6 +152,7 @@ StoreHandle HipExecuteContext::AssembleShards(int64_t local_device_id, int64_t g
       existing_store.has_value() ? *std::move(existing_store) : CreateStore(local_device_id, global_device_id, shape);
   require_live(output, "AssembleShards");
   std::lock_guard<std::mutex> lock(mu_);
+  FlushLocked();
   // across(shape.sharding.devices).if_on(p): only a member device copies its shard
   if (shape.sharding.devices.Contains(global_device_id)) {
     check(mmr_store_assemble(ctx_, output.impl->array->store, global_device_id, shard.data, shard.size, 2),
@@ -172,8 +174,25 @@ void HipExecuteContext::Reshard(int64_t local_device_id, int64_t global_device_i
   if (first) {
     op.a = s;
     op.b = d;
-    // the whole copy runs once, on the first arriving device's call
-    int rc = mmr_reshard(ctx_, src.impl->array->store, dst.impl->array->store);
+    // the whole copy runs once, for the first arriving device's call; it is queued so that the reshards of one
+    // schedule window leave in one batch
+    std::shared_ptr<SharedStore> sa = src.impl->array, da = dst.impl->array;
+    int rc = mmr_reshard_validate(ctx_, sa->store, da->store);
+    if (rc == MMR_OK && defer_reshards_) {
+      bool depends = false;
+      for (const auto& q : pending_)
+        depends |= q.second == sa || q.second == da || q.first == da;  // reads or overwrites a queued result / input
+      try {
+        if (depends) FlushLocked();
+      } catch (...) {
+        in_flight_["Reshard"].erase(seq);
+        next_seq_["Reshard"][local_device_id]--;
+        throw;
+      }
+      pending_.emplace_back(std::move(sa), std::move(da));
+    } else if (rc == MMR_OK) {
+      rc = mmr_reshard(ctx_, sa->store, da->store);
+    }
     if (rc != MMR_OK) {
       in_flight_["Reshard"].erase(seq);
       next_seq_["Reshard"][local_device_id]--;
@@ -186,9 +205,35 @@ void HipExecuteContext::Reshard(int64_t local_device_id, int64_t global_device_i
   Leave("Reshard", seq, op);
 }
 
+void HipExecuteContext::FlushLocked() {
+  if (pending_.empty()) return;
+  std::vector<mmr_store*> srcs, dsts;
+  for (const auto& q : pending_) {
+    srcs.push_back(q.first->store);
+    dsts.push_back(q.second->store);
+  }
+  auto keep = std::move(pending_);  // the stores stay alive until the launches are issued; a failure is not retried
+  pending_.clear();
+  check(srcs.size() == 1 ? mmr_reshard(ctx_, srcs[0], dsts[0])
+                         : mmr_reshard_batch(ctx_, srcs.data(), dsts.data(), static_cast<int32_t>(srcs.size())),
+        "Reshard");
+}
+
+void HipExecuteContext::Flush() {
+  std::lock_guard<std::mutex> lock(mu_);
+  FlushLocked();
+}
+
+void HipExecuteContext::SetDeferReshards(bool defer) {
+  std::lock_guard<std::mutex> lock(mu_);
+  FlushLocked();
+  defer_reshards_ = defer;
+}
+
 void* HipExecuteContext::SliceLocalShard(int64_t local_device_id, const StoreHandle& handle) {
   (void)local_device_id;
   require_live(handle, "SliceLocalShard");
+  Flush();
   void* ptr = nullptr;
   check(mmr_store_shard_ptr(ctx_, handle.impl->array->store, handle.impl->global_device_id, &ptr), "SliceLocalShard");
   return ptr;
@@ -196,6 +241,7 @@ void* HipExecuteContext::SliceLocalShard(int64_t local_device_id, const StoreHan
 
 void HipExecuteContext::CopyShardToHost(const StoreHandle& handle, void* host_dst, size_t size) {
   require_live(handle, "CopyShardToHost");
+  Flush();
   check(mmr_store_read_shard(ctx_, handle.impl->array->store, handle.impl->global_device_id, host_dst, size),
         "CopyShardToHost");
 }
@@ -242,6 +288,7 @@ void HipExecuteContext::OffloadDtoH(int64_t local_device_id, const std::vector<S
   const int64_t seq = next_seq_["OffloadDtoH"][local_device_id];
   ReplicatedOp& op = Arrive("OffloadDtoH", local_device_id, &first);
   if (first) {
+    FlushLocked();
     for (const StoreHandle& h : to_offload) {
       require_live(h, "OffloadDtoH");
       check(mmr_store_offload(ctx_, h.impl->array->store), "OffloadDtoH");
@@ -258,6 +305,7 @@ void HipExecuteContext::OffloadHtoD(int64_t local_device_id, const std::vector<S
   const int64_t seq = next_seq_["OffloadHtoD"][local_device_id];
   ReplicatedOp& op = Arrive("OffloadHtoD", local_device_id, &first);
   if (first) {
+    FlushLocked();
     for (const StoreHandle& h : to_offload) {
       require_live(h, "OffloadHtoD");
       check(mmr_store_reload(ctx_, h.impl->array->store), "OffloadHtoD");
@@ -266,10 +314,11 @@ void HipExecuteContext::OffloadHtoD(int64_t local_device_id, const std::vector<S
   Leave("OffloadHtoD", seq, op);
 }
 
-void HipExecuteContext::CloseWindow() {}
+void HipExecuteContext::CloseWindow() { Flush(); }
 
 void HipExecuteContext::RunAfterAllTasks(int64_t local_device_id, std::function<void()> on_done) {
   (void)local_device_id;
+  Flush();
   check(mmr_sync(ctx_), "RunAfterAllTasks");
   on_done();
 }
@@ -278,11 +327,13 @@ void HipExecuteContext::MarkProfile(const std::string& name) { (void)name; }
 
 void HipExecuteContext::StartTimer(const std::string& name) {
   (void)name;
+  Flush();
   check(mmr_timer_start(ctx_), "StartTimer");
 }
 
 void HipExecuteContext::StopTimer(const std::string& name) {
   float ms = 0;
+  Flush();
   check(mmr_timer_stop(ctx_, &ms), "StopTimer");
   timers_ms_[name] = ms;
 }
@@ -290,6 +341,7 @@ void HipExecuteContext::StopTimer(const std::string& name) {
 double HipExecuteContext::LastTimerMilliseconds(const std::string& name) { return timers_ms_[name]; }
 
 mmr_context_stats HipExecuteContext::Stats() {
+  Flush();
   mmr_context_stats s{};
   check(mmr_context_get_stats(ctx_, &s), "Stats");
   return s;

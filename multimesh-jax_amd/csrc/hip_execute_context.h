@@ -167,8 +167,20 @@ class HipExecuteContext {
   std::set<int> GetLocalDevices() { return local_devices_; }
   bool IsGpu() { return true; }
 
-  // Not part of the reference interface: inspection for tests and benchmarks.
-  mmr_context* raw() { return ctx_; }
+  // Reshard calls are queued and issued together - one plan, one launch per kernel class for a whole schedule
+  // window (the reference's Execute loop issues one Reshard per array, mm_pjrt_executable.cc:616-658; a pytree of
+  // 195 arrays is 195 calls).  The queue is flushed by every other entry point that touches device memory or
+  // time (AssembleShards, SliceLocalShard, CopyShardToHost, offloads, timers, RunAfterAllTasks, CloseWindow),
+  // by a Reshard that depends on a queued one, and by Flush().  An adapter that also runs compute tasks calls
+  // Flush() before it enqueues a task.  Argument errors are still raised by the Reshard call that causes them.
+  void Flush();
+  void SetDeferReshards(bool defer);
+
+  // Not part of the reference interface: inspection for tests and benchmarks (both flush first).
+  mmr_context* raw() {
+    Flush();
+    return ctx_;
+  }
   // What ToLiteral does through SliceLocalShard (mm_pjrt_buffer.cc:84-95): blocking copy of the handle's shard.
   void CopyShardToHost(const StoreHandle& handle, void* host_dst, size_t size);
   mmr_context_stats Stats();
@@ -187,7 +199,11 @@ class HipExecuteContext {
   ReplicatedOp& Arrive(const char* kind, int64_t local_device_id, bool* first);
   void Leave(const char* kind, int64_t seq, const ReplicatedOp& op);
 
+  void FlushLocked();
+
   mmr_context* ctx_{nullptr};
+  bool defer_reshards_{true};
+  std::vector<std::pair<std::shared_ptr<SharedStore>, std::shared_ptr<SharedStore>>> pending_;  // queued (src, dst)
   std::shared_ptr<std::atomic<bool>> alive_{std::make_shared<std::atomic<bool>>(true)};
   std::set<int> local_devices_;
   std::mutex mu_;

@@ -167,6 +167,76 @@ static int run() {
     EXPECT(throws([&] { ctx->Reshard(1, 1, root[1], param[1]); }, "control replication"));
   }
 
+  // A schedule window of many Reshard ops (a pytree crossing a task boundary, mm_pjrt_executable.cc:616-658):
+  // op by op, device by device, exactly as Execute issues them.  They leave as one batch: one plan, one launch.
+  {
+    auto win = HipExecuteContext::Create(local);
+    const int kArrays = 9;
+    std::vector<ShardedShape> ws(kArrays), wd(kArrays);
+    std::vector<std::vector<std::vector<float>>> wshards(kArrays);
+    std::vector<std::vector<StoreHandle>> wparam(kArrays, std::vector<StoreHandle>(kLocal)),
+        wroot(kArrays, std::vector<StoreHandle>(kLocal));
+    for (int a = 0; a < kArrays; ++a) {
+      const int64_t rows = 64 * (1 + a % 3), cols = 128 * (1 + a % 2);
+      ws[a] = ShardedShape{SupportedType::F32, {{{rows, 1, 0}, {cols, 4, 1}}, DeviceList::Create(0, 4)}, {}};
+      wd[a] = ShardedShape{SupportedType::F32, {{{rows, 8, 0}, {cols, 1, 1}}, DeviceList::Create(4, 8)}, {}};
+      wshards[a].assign(4, std::vector<float>(rows * cols / 4));
+      for (auto& sh : wshards[a])
+        for (auto& v : sh) {
+          lcg = lcg * 1664525u + 1013904223u;
+          v = static_cast<float>(lcg >> 8);
+        }
+      for (int d = 0; d < kLocal; ++d) {
+        Shard shard{d < 4 ? wshards[a][d].data() : nullptr, d, d < 4 ? wshards[a][d].size() * 4 : 0};
+        wparam[a][d] = win->AssembleShards(d, d, ws[a], shard);
+      }
+      for (int d = 0; d < kLocal; ++d) wroot[a][d] = win->CreateStore(d, d, wd[a]);
+    }
+    const mmr_context_stats before = win->Stats();
+    for (int a = 0; a < kArrays; ++a)
+      for (int d = 0; d < kLocal; ++d) win->Reshard(d, d, wparam[a][d], wroot[a][d]);
+    const mmr_context_stats after = win->Stats();  // flushes the window
+    EXPECT(after.reshard_calls - before.reshard_calls == 1);
+    EXPECT(after.kernel_launches - before.kernel_launches == 1);
+    EXPECT(after.plans_built - before.plans_built == 1);
+    for (int a = 0; a < kArrays; ++a) {
+      const size_t n = static_cast<size_t>(ShardSize(wd[a])) / 4;
+      std::vector<std::vector<float>> want(8, std::vector<float>(n));
+      orc_desc so = to_orc(ws[a], 4), dd = to_orc(wd[a], 4);
+      const void* sp[4];
+      void* dp[8];
+      for (int k = 0; k < 4; ++k) sp[k] = wshards[a][k].data();
+      for (int k = 0; k < 8; ++k) dp[k] = want[k].data();
+      EXPECT(orc_reshard(&so, sp, &dd, dp, 1) == 0);
+      for (int d = 4; d < kLocal; ++d) {
+        std::vector<float> got(n);
+        win->CopyShardToHost(wroot[a][d], got.data(), n * 4);
+        EXPECT(std::memcmp(got.data(), want[d - 4].data(), n * 4) == 0);
+      }
+    }
+    // a chain inside one window (B := reshard(A), then A2 := reshard(B)) is split where it depends on itself
+    std::vector<StoreHandle> back(kLocal);
+    for (int d = 0; d < kLocal; ++d) back[d] = win->CreateStore(d, d, ws[0]);
+    const mmr_context_stats b2 = win->Stats();
+    for (int d = 0; d < kLocal; ++d) win->Reshard(d, d, wparam[0][d], wroot[0][d]);
+    for (int d = 0; d < kLocal; ++d) win->Reshard(d, d, wroot[0][d], back[d]);
+    const mmr_context_stats a2 = win->Stats();
+    EXPECT(a2.reshard_calls - b2.reshard_calls == 2);
+    for (int d = 0; d < 4; ++d) {
+      std::vector<float> got(wshards[0][d].size());
+      win->CopyShardToHost(back[d], got.data(), got.size() * 4);
+      EXPECT(std::memcmp(got.data(), wshards[0][d].data(), got.size() * 4) == 0);  // round trip restores the source
+    }
+    // a bad call is reported by the call itself, not when the window is flushed
+    EXPECT(throws([&] { win->Reshard(0, 0, wparam[0][0], wroot[1][0]); }, "in the source and"));
+    // without deferral every op launches on its own
+    win->SetDeferReshards(false);
+    const mmr_context_stats b3 = win->Stats();
+    for (int a = 0; a < 3; ++a)
+      for (int d = 0; d < kLocal; ++d) win->Reshard(d, d, wparam[a][d], wroot[a][d]);
+    EXPECT(win->Stats().reshard_calls - b3.reshard_calls == 3);
+  }
+
   // Free(keep_in_cache) + CreateStore(allocate_from_cache) on a fresh context
   auto ctx2 = HipExecuteContext::Create({0, 1});
   ShardedShape small{SupportedType::F32, {{{16, 2, 0}}, DeviceList::Create(0, 2)}, {}};
