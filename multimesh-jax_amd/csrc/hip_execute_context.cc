@@ -347,4 +347,60 @@ mmr_context_stats HipExecuteContext::Stats() {
   return s;
 }
 
+Store ReshardSchedule::AddStore(Store::Type type, std::string name, ShardedShape shape) {
+  Store store;
+  store.type = type;
+  store.name = std::move(name);
+  store.sharded_shape = std::move(shape);
+  switch (type) {
+    case Store::Type::PARAM: store.index = num_params_++; break;
+    case Store::Type::ROOT: store.index = num_roots_++; break;
+    case Store::Type::TEMP:
+      store.index = static_cast<int64_t>(temporaries_.size());
+      temporaries_.push_back(store);
+      break;
+  }
+  return store;
+}
+
+void ReshardSchedule::AddReshardTask(const Store& input, const Store& output) {
+  if (output.type == Store::Type::PARAM) raise("AddReshardTask: a parameter store cannot be a reshard's output");
+  if (!already_scheduled_.emplace(input.name, output.name).second) return;
+  schedule_.push_back(MpmdOperation{Reshard{input, output}});
+}
+
+std::vector<std::vector<StoreHandle>> ReshardSchedule::Execute(
+    HipExecuteContext& ctx, const std::vector<std::vector<StoreHandle>>& parameter_stores) {
+  const std::set<int> local = ctx.GetLocalDevices();
+  const std::vector<int> devices(local.begin(), local.end());
+  const size_t n = devices.size();
+  if (parameter_stores.size() != n) raise("Execute: one list of parameter stores per local device is required");
+  for (const auto& p : parameter_stores)
+    if (static_cast<int64_t>(p.size()) != num_params_) raise("Execute: wrong number of parameter stores");
+  std::vector<std::vector<StoreHandle>> root_stores(n, std::vector<StoreHandle>(static_cast<size_t>(num_roots_)));
+  for (const MpmdOperation& op : schedule_) {  // add_root_store: once per root, for every local device
+    const Store& out = op.op.output;
+    if (out.type != Store::Type::ROOT || root_stores[0][out.index].impl) continue;
+    for (size_t i = 0; i < n; ++i)
+      root_stores[i][out.index] = ctx.CreateStore(devices[i], devices[i], out.sharded_shape, {.name = out.name});
+  }
+  if (cached_temporary_stores_.empty()) {
+    cached_temporary_stores_.resize(n);
+    for (size_t i = 0; i < n; ++i)
+      for (const Store& t : temporaries_)
+        cached_temporary_stores_[i].push_back(ctx.CreateStore(devices[i], devices[i], t.sharded_shape, {.name = t.name}));
+  }
+  auto handle_of = [&](size_t i, const Store& store) -> const StoreHandle& {
+    switch (store.type) {
+      case Store::Type::PARAM: return parameter_stores[i][store.index];
+      case Store::Type::ROOT: return root_stores[i][store.index];
+      default: return cached_temporary_stores_[i][store.index];
+    }
+  };
+  for (const MpmdOperation& op : schedule_)
+    for (size_t i = 0; i < n; ++i)
+      ctx.Reshard(devices[i], devices[i], handle_of(i, op.op.input), handle_of(i, op.op.output));
+  return root_stores;
+}
+
 }  // namespace mmr

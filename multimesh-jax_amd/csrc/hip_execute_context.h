@@ -213,6 +213,38 @@ class HipExecuteContext {
   friend struct StoreHandleImpl;
 };
 
+// mpmd_partition.h:40-55 without the compute task: what a schedule holds on this path.
+struct MpmdOperation {
+  Reshard op;
+};
+
+// The reshard part of a compiled schedule and of its execution:
+//   * AddStore / AddReshardTask as MpmdScheduler does (mpmd_partition.cc:250-323, 340-351): stores are named,
+//     typed PARAM / ROOT / TEMP and indexed per type; a reshard is scheduled once;
+//   * Execute as MultiMeshPjRtExecutable::Execute does (mm_pjrt_executable.cc:470-561 store set-up, 592-658 loop):
+//     a fresh ROOT store per reshard output of type ROOT and execution, TEMP stores created on the first execution
+//     and reused afterwards (cached_temporary_stores_), then every op issued by every local device in turn.
+// Compute tasks are not part of it; the reshards of the whole schedule leave as one window.
+class ReshardSchedule {
+ public:
+  Store AddStore(Store::Type type, std::string name, ShardedShape shape);
+  void AddReshardTask(const Store& input, const Store& output);
+  const std::vector<MpmdOperation>& schedule() const { return schedule_; }
+  int64_t num_parameters() const { return num_params_; }
+  int64_t num_roots() const { return num_roots_; }
+  // parameter_stores[local device position][parameter index] -> root_stores[local device position][root index];
+  // positions follow the order of ctx.GetLocalDevices().
+  std::vector<std::vector<StoreHandle>> Execute(HipExecuteContext& ctx,
+                                                const std::vector<std::vector<StoreHandle>>& parameter_stores);
+
+ private:
+  std::vector<MpmdOperation> schedule_;
+  std::set<std::pair<std::string, std::string>> already_scheduled_;
+  std::vector<Store> temporaries_;
+  int64_t num_params_{0}, num_roots_{0};
+  std::vector<std::vector<StoreHandle>> cached_temporary_stores_;  // [local device position][temp index]
+};
+
 }  // namespace mmr
 
 #endif  // MMR_CSRC_HIP_EXECUTE_CONTEXT_H_

@@ -237,6 +237,71 @@ static int run() {
     EXPECT(win->Stats().reshard_calls - b3.reshard_calls == 3);
   }
 
+  // The schedule mirror: stores and reshard tasks registered as the scheduler does, executed as Execute does.
+  {
+    auto sc = HipExecuteContext::Create(local);
+    ShardedShape a{SupportedType::F32, {{{96, 1, 0}, {128, 4, 1}}, DeviceList::Create(0, 4)}, {}};
+    ShardedShape b{SupportedType::F32, {{{96, 8, 0}, {128, 1, 1}}, DeviceList::Create(4, 8)}, {}};
+    ShardedShape c{SupportedType::F32, {{{96, 2, 0}, {128, 2, 1}}, DeviceList::Create(0, 4)}, {}};
+    ReshardSchedule schedule;
+    Store p0 = schedule.AddStore(Store::Type::PARAM, "p0", a);
+    Store p1 = schedule.AddStore(Store::Type::PARAM, "p1", a);
+    Store t0 = schedule.AddStore(Store::Type::TEMP, "t0", b);
+    Store r0 = schedule.AddStore(Store::Type::ROOT, "r0", c);
+    Store r1 = schedule.AddStore(Store::Type::ROOT, "r1", b);
+    schedule.AddReshardTask(p0, t0);
+    schedule.AddReshardTask(t0, r0);  // depends on the first: the window splits here
+    schedule.AddReshardTask(p1, r1);
+    schedule.AddReshardTask(p1, r1);  // scheduled once
+    EXPECT(schedule.schedule().size() == 3 && schedule.num_parameters() == 2 && schedule.num_roots() == 2);
+    std::vector<std::vector<float>> data0(4, std::vector<float>(96 * 32)), data1 = data0;
+    for (auto* set : {&data0, &data1})
+      for (auto& sh : *set)
+        for (auto& v : sh) {
+          lcg = lcg * 1664525u + 1013904223u;
+          v = static_cast<float>(lcg >> 9);
+        }
+    std::vector<std::vector<StoreHandle>> params(kLocal, std::vector<StoreHandle>(2));
+    for (int d = 0; d < kLocal; ++d) {
+      params[d][0] = sc->AssembleShards(d, d, a, Shard{d < 4 ? data0[d].data() : nullptr, d, d < 4 ? data0[d].size() * 4 : 0});
+      params[d][1] = sc->AssembleShards(d, d, a, Shard{d < 4 ? data1[d].data() : nullptr, d, d < 4 ? data1[d].size() * 4 : 0});
+    }
+    auto expect_for = [&](const std::vector<std::vector<float>>& in, const ShardedShape& to, int devs) {
+      std::vector<std::vector<float>> out(devs, std::vector<float>(static_cast<size_t>(ShardSize(to)) / 4));
+      orc_desc so = to_orc(a, 4), dd = to_orc(to, 4);
+      const void* sp[4];
+      void* dp[8];
+      for (int k = 0; k < 4; ++k) sp[k] = in[k].data();
+      for (int k = 0; k < devs; ++k) dp[k] = out[k].data();
+      if (orc_reshard(&so, sp, &dd, dp, 1) != 0) out.clear();
+      return out;
+    };
+    const auto want_r0 = expect_for(data0, c, 4), want_r1 = expect_for(data1, b, 8);
+    EXPECT(!want_r0.empty() && !want_r1.empty());
+    int64_t first_root = -1;
+    const int64_t stores_before = sc->Stats().stores_live;
+    for (int run_index = 0; run_index < 2; ++run_index) {
+      const mmr_context_stats s0 = sc->Stats();
+      auto roots = schedule.Execute(*sc, params);
+      const mmr_context_stats s1 = sc->Stats();
+      EXPECT(s1.reshard_calls - s0.reshard_calls == 2);  // {p0->t0} | {t0->r0, p1->r1}
+      for (int d = 0; d < 4; ++d) {
+        std::vector<float> got(want_r0[d].size());
+        sc->CopyShardToHost(roots[d][0], got.data(), got.size() * 4);
+        EXPECT(std::memcmp(got.data(), want_r0[d].data(), got.size() * 4) == 0);
+      }
+      for (int d = 4; d < kLocal; ++d) {
+        std::vector<float> got(want_r1[d - 4].size());
+        sc->CopyShardToHost(roots[d][1], got.data(), got.size() * 4);
+        EXPECT(std::memcmp(got.data(), want_r1[d - 4].data(), got.size() * 4) == 0);
+      }
+      // roots are new stores per execution, the temporary is created once
+      if (run_index == 0) first_root = roots[0][0].unique_id;
+      else EXPECT(roots[0][0].unique_id != first_root);
+      EXPECT(sc->Stats().stores_live == stores_before + 1 + 2);  // t0 + this run's two roots (last run's are gone)
+    }
+  }
+
   // Free(keep_in_cache) + CreateStore(allocate_from_cache) on a fresh context
   auto ctx2 = HipExecuteContext::Create({0, 1});
   ShardedShape small{SupportedType::F32, {{{16, 2, 0}}, DeviceList::Create(0, 2)}, {}};
