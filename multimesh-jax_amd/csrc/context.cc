@@ -41,6 +41,15 @@ struct DevicePlan {
   };
   std::vector<TransposeRun> transpose_runs;  // the table is sorted by itemsize; one launch per run
   bool tuned = false;                        // the table order has been chosen (timed or fixed by the options)
+
+  DevicePlan() = default;
+  DevicePlan(const DevicePlan&) = delete;
+  DevicePlan& operator=(const DevicePlan&) = delete;
+  ~DevicePlan() {  // hipFree waits for the device: launches that still read the tables finish first
+    (void)hipFree(d_copy16);
+    (void)hipFree(d_generic);
+    (void)hipFree(d_transposes);
+  }
 };
 
 struct Binding {
@@ -130,14 +139,6 @@ void drop_bindings_of(mmr_context* ctx, int64_t store_id) {
   }
 }
 
-void free_tables(DevicePlan* dp) {
-  (void)hipFree(dp->d_copy16);
-  (void)hipFree(dp->d_generic);
-  (void)hipFree(dp->d_transposes);
-  dp->d_copy16 = dp->d_generic = nullptr;
-  dp->d_transposes = nullptr;
-}
-
 // Plans n descriptor pairs under `options` and uploads the tables (not cached here).
 int make_device_plan(mmr_context* ctx, const std::vector<mmr_sharded_shape>& srcs, const std::vector<mmr_sharded_shape>& dsts,
                      const mmr_plan_options& options, DevicePlan* dp) {
@@ -173,10 +174,7 @@ int get_plan(mmr_context* ctx, const std::vector<mmr_sharded_shape>& srcs, const
     return MMR_OK;
   }
   auto dp = std::make_unique<DevicePlan>();
-  if (int rc = make_device_plan(ctx, srcs, dsts, ctx->options, dp.get())) {
-    free_tables(dp.get());
-    return rc;
-  }
+  if (int rc = make_device_plan(ctx, srcs, dsts, ctx->options, dp.get())) return rc;
   ctx->stats.plans_built += 1;
   *out = dp.get();
   ctx->plans.emplace(std::move(key), std::move(dp));
@@ -251,25 +249,18 @@ int tune_plan(mmr_context* ctx, DevicePlan* dp, void* const* d_ptrs) {
     if (rc == MMR_OK) timed += 1;
     if (rc == MMR_OK && ms < 0.98f * best_ms) {  // only a clear win replaces the default
       best_ms = ms;
-      if (best) free_tables(best.get());
       best = std::move(alt);
-    } else {
-      (void)hipStreamSynchronize(ctx->stream);
-      free_tables(alt.get());
     }
   }
   (void)hipEventDestroy(e0);
   (void)hipEventDestroy(e1);
-  if (rc == MMR_OK && best) {  // the cached object keeps its address: bindings point at it
-    free_tables(dp);
-    dp->plan = std::move(best->plan);
-    dp->d_copy16 = best->d_copy16;
-    dp->d_generic = best->d_generic;
-    dp->d_transposes = best->d_transposes;
-    dp->transpose_runs = std::move(best->transpose_runs);
+  if (rc == MMR_OK && best) {  // the cached object keeps its address (bindings point at it) and takes the winner's tables
+    std::swap(dp->plan, best->plan);
+    std::swap(dp->d_copy16, best->d_copy16);
+    std::swap(dp->d_generic, best->d_generic);
+    std::swap(dp->d_transposes, best->d_transposes);
+    std::swap(dp->transpose_runs, best->transpose_runs);
     dp->plan.options = base;  // still the plan of the context's options
-  } else if (best) {
-    free_tables(best.get());
   }
   dp->plan.stats.orders_timed = timed;
   return rc;
@@ -396,11 +387,7 @@ void mmr_context_destroy(mmr_context* ctx) {
   (void)hipSetDevice(ctx->device);
   (void)hipStreamSynchronize(ctx->stream);
   for (auto& b : ctx->bindings) (void)hipFree(b.second->d_ptrs);
-  for (auto& p : ctx->plans) {
-    (void)hipFree(p.second->d_copy16);
-    (void)hipFree(p.second->d_generic);
-    (void)hipFree(p.second->d_transposes);
-  }
+  ctx->plans.clear();
   for (auto& s : ctx->stores) {
     (void)hipFree(s.second->base);
     if (s.second->host) (void)hipHostFree(s.second->host);
