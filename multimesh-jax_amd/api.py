@@ -324,8 +324,9 @@ class ReshardContext:
         return StoreHandle(self, h, shape, name or "anonymous")
 
     def AssembleShards(self, shape: B.ShardedShape, device: int, data, existing_store: Optional[StoreHandle] = None,
-                       size: Optional[int] = None) -> StoreHandle:
-        """Shard{data, local_device_id, size}: `data` is a NumPy array (host) or an int device pointer."""
+                       size: Optional[int] = None, where: int = 1) -> StoreHandle:
+        """Shard{data, local_device_id, size}: `data` is a NumPy array (host) or an int pointer; `where` says what an
+        int pointer points at: 1 device memory, 0 host memory, 2 let the runtime find out."""
         store = existing_store if existing_store is not None else self.CreateStore(shape)
         if isinstance(data, np.ndarray):
             arr = np.ascontiguousarray(data)
@@ -333,7 +334,7 @@ class ReshardContext:
         else:
             if size is None:
                 raise ValueError("size is required for a device pointer")
-            B.check(self._lib.mmr_store_assemble(self._h, store._h, device, C.c_void_p(int(data)), size, 1))
+            B.check(self._lib.mmr_store_assemble(self._h, store._h, device, C.c_void_p(int(data)), size, where))
         return store
 
     def AdoptShards(self, shape: B.ShardedShape, device_ptrs: Sequence[int], name: Optional[str] = None) -> StoreHandle:

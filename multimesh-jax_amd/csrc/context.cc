@@ -507,6 +507,14 @@ int mmr_store_assemble(mmr_context* ctx, mmr_store* store, int64_t device, const
                              : data_on_device == 0 ? hipMemcpyHostToDevice
                                                    : hipMemcpyDefault;  // the runtime looks the pointer up
   if (store->offloaded()) return fail(MMR_INVALID_ARGUMENT, "store %lld is offloaded to host memory", (long long)store->id);
+  if (data_on_device == 2 && size >= (1u << 20)) {  // worth asking the runtime where the pointer lives
+    hipPointerAttribute_t attr{};
+    if (hipPointerGetAttributes(&attr, data) == hipSuccess) {
+      if (attr.type == hipMemoryTypeDevice && attr.device == ctx->device) data_on_device = 1;
+    } else {
+      (void)hipGetLastError();  // plain host memory is unknown to the runtime: not an error here
+    }
+  }
   // a large device-resident shard goes through the library's own copy kernel (6.4 TB/s against 5.3 TB/s for the
   // runtime's device-to-device copy on MI355X); anything else through the runtime
   const uintptr_t bits = reinterpret_cast<uintptr_t>(data) | reinterpret_cast<uintptr_t>(store->tile(k));

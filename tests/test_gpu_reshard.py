@@ -539,6 +539,14 @@ def test_device_resident_shards_assemble_through_the_copy_kernel(ctx):
         got = ctx.ReadShard(dst, 1)
         assert got[:size].tobytes() == data[:size].tobytes(), size
         assert (got[size:] == 0x77).all(), size
+    # a caller that does not say where the pointer lives (the C++ mirror): the runtime is asked, device memory still
+    # takes the kernel, host memory the runtime's copy
+    before = ctx.stats["kernel_launches"]
+    ctx.AssembleShards(shape, 1, ptr, existing_store=dst, size=n, where=2)
+    ctx.AssembleShards(shape, 0, data.ctypes.data, existing_store=dst, size=n, where=2)
+    ctx.Sync()
+    assert ctx.stats["kernel_launches"] - before == 1
+    assert ctx.ReadShard(dst, 1).tobytes() == data.tobytes() and ctx.ReadShard(dst, 0).tobytes() == data.tobytes()
     # rate of the device-to-device assemble
     reps = 20
     ctx.Sync()
