@@ -223,19 +223,26 @@ MMR_HD void generic_rows(const mmr_copy_chunk& c, typename M::cptr src, typename
     }
     return;
   }
-  const uint32_t R = THREADS / slots;
-  const uint32_t sub = tid / slots;
-  const uint32_t slot = tid - sub * slots;
-  if (sub >= R) return;
-  for (uint32_t row0 = sub; row0 < rows; row0 += R * UNROLL) {
+  // Rows narrower than the workgroup: the (row, slot) pairs of the chunk are numbered row after row and dealt to
+  // the lanes without regard to row ends, so no lane idles while pairs are left.  One division per thread; after
+  // that a lane's pair advances by THREADS pairs per step = (step_rows, step_slots) with a carry.
+  const uint32_t total = rows * slots;
+  const uint32_t step_rows = THREADS / slots, step_slots = THREADS - step_rows * slots;
+  uint32_t row = tid / slots, slot = tid - row * slots;
+  for (uint32_t i0 = tid; i0 < total; i0 += THREADS * UNROLL) {
     V16 v[UNROLL];
     typename M::ptr dpos[UNROLL];
     int32_t len[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       len[u] = 0;
-      const uint32_t row = row0 + u * R;
-      if (row < rows) generic_load<M, WIDE>(c, src, dst, fill, row, slot, &v[u], &dpos[u], &len[u]);
+      if (i0 + u * THREADS < total) generic_load<M, WIDE>(c, src, dst, fill, row, slot, &v[u], &dpos[u], &len[u]);
+      row += step_rows;
+      slot += step_slots;
+      if (slot >= slots) {
+        slot -= slots;
+        row += 1;
+      }
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) generic_store<M, WIDE>(dpos[u], len[u], v[u]);
