@@ -132,6 +132,13 @@ int mmr_needs_reshard(int64_t operand_dev_start, int64_t operand_dev_count, int6
                       int64_t dev_count, const mmr_op_sharding* operand_sharding,
                       const mmr_op_sharding* sharding, int32_t* out);
 
+/* ToMpmdSharding, mpmd_partition.cc:128-166: a sharding written relative to a task's devices (ids 0..n-1, as it
+ * stands inside the task's module) -> the sharding over global device ids.  rank = tensor rank.  An explicit
+ * device list or a single device is written to devices_out (capacity entries) and out points at it. */
+int mmr_to_mpmd_sharding(int32_t rank, const mmr_op_sharding* sharding, int64_t task_dev_start, int64_t task_dev_count,
+                         int64_t global_dev_start, int64_t global_dev_count, mmr_op_sharding* out, int64_t* devices_out,
+                         int64_t devices_capacity);
+
 /* Shard geometry: what spmd::MakePartitionedShape + ByteSizeOfElements give the
  * plugin (mm_pjrt_executable.cc:537, mm_pjrt_buffer.cc:285-288) and what the
  * mock calls zuku::ShardSize (mm_mock_mm_xla.cc:75). */

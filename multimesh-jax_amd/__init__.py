@@ -8,7 +8,7 @@ from . import _binding
 from ._binding import LIB_PATH, MmrError, load  # noqa: F401
 from .api import (  # noqa: F401
     CanonicalizeSharding, ComputeGlobalIndex, ComputeIndexSet, LogicalShardingToOpSharding, LogicalToPhysicalSharding,
-    MeshEquivalentSharding, NeedsReshard, Plan, ReshardContext, StoreHandle, TileAssignmentDevices,
+    MeshEquivalentSharding, NeedsReshard, Plan, ReshardContext, StoreHandle, TileAssignmentDevices, ToMpmdSharding,
     XlaShapeToZukuShape, describe, device_of_tile, itemsize, op_sharding, partition_spec_to_sharded_shape, shard_bytes,
     shard_extents,
     sharded_shape, tile_of_device,

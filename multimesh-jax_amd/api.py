@@ -181,6 +181,19 @@ def NeedsReshard(operand_devices: Tuple[int, int], devices: Tuple[int, int], ope
     return bool(out.value)
 
 
+def ToMpmdSharding(rank: int, sharding: B.OpSharding, task_devices: Tuple[int, int],
+                   global_devices: Tuple[int, int]) -> B.OpSharding:
+    """A sharding written relative to a task's devices -> the sharding over global device ids
+    (mpmd_partition.cc:128-166).  Device ranges are (start, count)."""
+    out = B.OpSharding()
+    n = max(int(sharding.n_devices), 1)
+    devices = _i64([0] * n)
+    B.check(B.load().mmr_to_mpmd_sharding(rank, C.byref(sharding), task_devices[0], task_devices[1], global_devices[0],
+                                          global_devices[1], C.byref(out), devices, n))
+    out._keepalive = devices
+    return out
+
+
 def shard_extents(s: B.ShardedShape) -> Tuple[int, ...]:
     ext = _i64([0] * B.MMR_MAX_DIMS)
     rank = C.c_int32()

@@ -417,4 +417,65 @@ int mmr_needs_reshard(int64_t operand_dev_start, int64_t operand_dev_count, int6
   return MMR_OK;
 }
 
+int mmr_to_mpmd_sharding(int32_t rank, const mmr_op_sharding* sharding, int64_t task_dev_start, int64_t task_dev_count,
+                         int64_t global_dev_start, int64_t global_dev_count, mmr_op_sharding* out, int64_t* devices_out,
+                         int64_t devices_capacity) {
+  if (int rc = check_sharding(sharding)) return rc;
+  if (!out) return fail(MMR_INVALID_ARGUMENT, "null output");
+  if (rank < 0 || rank >= MMR_MAX_DIMS) return fail(MMR_INVALID_ARGUMENT, "rank %d", rank);
+  if (task_dev_count < 1) return fail(MMR_INVALID_ARGUMENT, "empty task device list");
+  mmr_op_sharding r{};
+  const bool same_devices = task_dev_start == global_dev_start && task_dev_count == global_dev_count;
+  // :132-134  replicated over the whole machine stays replicated
+  if (is_replicated(*sharding) && same_devices) {
+    r.type = MMR_SHARDING_REPLICATED;
+    *out = r;
+    return MMR_OK;
+  }
+  // :136-139  one device: the array lives on that device
+  if (task_dev_count == 1 && (is_maximal(*sharding) || is_replicated(*sharding))) {
+    if (!devices_out || devices_capacity < 1) return fail(MMR_INVALID_ARGUMENT, "device list output too small");
+    devices_out[0] = task_dev_start;
+    r.type = MMR_SHARDING_MAXIMAL;
+    r.tile_assignment_devices = devices_out;
+    r.n_devices = 1;
+    *out = r;
+    return MMR_OK;
+  }
+  r = *sharding;
+  r.tile_assignment_devices = nullptr;
+  r.n_devices = 0;
+  if (sharding->n_iota_dims > 0) {
+    r.iota_offset = task_dev_start;  // :143-144
+  } else if (sharding->n_devices > 0) {
+    // :145-150  ids relative to the task's device list -> global ids
+    if (!devices_out || devices_capacity < sharding->n_devices)
+      return fail(MMR_INVALID_ARGUMENT, "device list output too small");
+    for (int64_t i = 0; i < sharding->n_devices; ++i) {
+      const int64_t rel = sharding->tile_assignment_devices[i];
+      if (rel < 0 || rel >= task_dev_count)
+        return fail(MMR_INVALID_ARGUMENT, "relative device id %lld outside the task's %lld devices", (long long)rel,
+                    (long long)task_dev_count);
+      devices_out[i] = task_dev_start + rel;
+    }
+    r.tile_assignment_devices = devices_out;
+    r.n_devices = sharding->n_devices;
+  }
+  // :152-163  replicated on a subset of the devices: one tile per tensor dim, all of the task's devices as replicas
+  if (is_replicated(*sharding) && rank > 0) {
+    r = mmr_op_sharding{};
+    r.type = MMR_SHARDING_OTHER;
+    r.n_tile_dims = rank + 1;
+    for (int i = 0; i < rank; ++i) r.tile_dims[i] = 1;
+    r.tile_dims[rank] = task_dev_count;
+    r.n_iota_dims = 1;
+    r.iota_reshape_dims[0] = task_dev_count;
+    r.iota_transpose_perm[0] = 0;
+    r.iota_offset = task_dev_start;
+    r.replicate_on_last_tile_dim = 1;
+  }
+  *out = r;
+  return MMR_OK;
+}
+
 }  // extern "C"

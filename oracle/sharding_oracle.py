@@ -24,6 +24,10 @@ tests, re-expressed as numbers in tests/golden/sharding_golden.json:
       190-205 expects (3 active cases, exact fields) and :116-187 (2 cases the
       reference skips; given in XLA's canonical form, compared as tile dims
       plus device order)
+  to_mpmd_sharding
+      src/pjrt_client/mpmd_partition.cc:128-166
+      pinned by the store shardings mpmd_partition_test.cc:1381-1418 and
+      :1455-1484 expect (rebased iota offsets; replication on a submesh)
   canonicalize_sharding
       src/pjrt_client/mm_sharding.cc:275-456
       pinned by mm_sharding_test.cc:529-737 (3 golden descriptors, 1 error)
@@ -432,3 +436,29 @@ def needs_reshard(operand_devices: Tuple[int, int], devices: Tuple[int, int],
         return False
     return tuple(operand_devices) != tuple(devices) or not mesh_equivalent_sharding(
         operand_sharding, sharding)
+
+
+def to_mpmd_sharding(rank: int, sharding: OpSharding, task_devices: Tuple[int, int],
+                     global_devices: Tuple[int, int]) -> OpSharding:
+    """mpmd_partition.cc:128-166.  `sharding` is written relative to the task's devices (ids 0..n-1); the result
+    names global device ids.  Device ranges are (start, count)."""
+    t_start, t_count = task_devices
+    if sharding.type == "REPLICATED" and tuple(task_devices) == tuple(global_devices):   # :132-134
+        return OpSharding(type="REPLICATED")
+    if t_count == 1 and sharding.type in ("MAXIMAL", "REPLICATED"):                       # :136-139
+        return OpSharding(type="MAXIMAL", tile_assignment_devices=[t_start])
+    if sharding.type == "REPLICATED" and rank > 0:                                         # :152-163
+        return OpSharding(type="OTHER", tile_assignment_dimensions=[1] * rank + [t_count], iota_reshape_dims=[t_count],
+                          iota_transpose_perm=[0], replicate_on_last_tile_dim=True, iota_offset=t_start)
+    out = OpSharding(type=sharding.type, tile_assignment_dimensions=list(sharding.tile_assignment_dimensions),
+                     iota_reshape_dims=list(sharding.iota_reshape_dims),
+                     iota_transpose_perm=list(sharding.iota_transpose_perm),
+                     replicate_on_last_tile_dim=sharding.replicate_on_last_tile_dim, iota_offset=sharding.iota_offset)
+    if sharding.has_iota:
+        out.iota_offset = t_start                                                          # :143-144
+    else:
+        for rel in sharding.tile_assignment_devices:                                        # :145-150
+            if not 0 <= rel < t_count:
+                raise ShardingError("relative device id %d outside the task's %d devices" % (rel, t_count))
+        out.tile_assignment_devices = [t_start + rel for rel in sharding.tile_assignment_devices]
+    return out

@@ -280,3 +280,54 @@ def test_logical_sharding_known_answers_of_the_reference():
                                                   e["replicate_on_last_tile_dim"]), c["source"]
         for k in e:
             assert got[k] == e[k], (c["source"], k)
+
+
+def _lib_op2(d):
+    return mm.op_sharding(d["type"], d.get("tile_dims", ()), d.get("iota_reshape_dims", ()),
+                          d.get("iota_transpose_perm", ()), d.get("tile_assignment_devices", ()),
+                          d.get("replicate_on_last_tile_dim", False), d.get("iota_offset", 0))
+
+
+def _oracle_op2(d):
+    return so.OpSharding(type=d["type"], tile_assignment_dimensions=list(d.get("tile_dims", [])),
+                         iota_reshape_dims=list(d.get("iota_reshape_dims", [])),
+                         iota_transpose_perm=list(d.get("iota_transpose_perm", [])),
+                         tile_assignment_devices=list(d.get("tile_assignment_devices", [])),
+                         replicate_on_last_tile_dim=d.get("replicate_on_last_tile_dim", False),
+                         iota_offset=d.get("iota_offset", 0))
+
+
+def test_to_mpmd_sharding_known_answers_of_the_reference(golden):
+    """Store shardings mpmd_partition_test.cc expects after ToMpmdSharding (iota offsets rebased to the task's
+    devices, replication on a submesh spelled out), for the oracle restatement and the C ABI."""
+    cases = golden["to_mpmd_sharding"]
+    assert len(cases) >= 4
+    for c in cases:
+        e = c["expect"]
+        o = so.to_mpmd_sharding(c["rank"], _oracle_op2(c["sharding"]), tuple(c["task_devices"]), tuple(c["global_devices"]))
+        assert (o.type, o.tile_assignment_dimensions, o.iota_reshape_dims, o.iota_transpose_perm, o.iota_offset,
+                o.replicate_on_last_tile_dim) == (e["type"], e["tile_dims"], e["iota_reshape_dims"],
+                                                  e["iota_transpose_perm"], e["iota_offset"],
+                                                  e["replicate_on_last_tile_dim"]), c["source"]
+        got = _op_dict(mm.ToMpmdSharding(c["rank"], _lib_op2(c["sharding"]), tuple(c["task_devices"]),
+                                         tuple(c["global_devices"])))
+        for k in e:
+            assert got[k] == e[k], (c["source"], k)
+
+
+def test_to_mpmd_sharding_special_cases():
+    """The branches no reference test exercises, from what they must mean: replication over the whole machine stays
+    replication; on a single device the array lives on that device; relative device ids become global ones."""
+    rep = mm.op_sharding("REPLICATED")
+    assert _op_dict(mm.ToMpmdSharding(2, rep, (0, 8), (0, 8)))["type"] == "REPLICATED"
+    one = mm.ToMpmdSharding(2, rep, (5, 1), (0, 8))
+    assert _op_dict(one)["type"] == "MAXIMAL" and one.n_devices == 1 and one.tile_assignment_devices[0] == 5
+    listed = mm.op_sharding("OTHER", [2, 2], tile_assignment_devices=[0, 2, 1, 3])
+    out = mm.ToMpmdSharding(2, listed, (4, 4), (0, 8))
+    assert [out.tile_assignment_devices[i] for i in range(out.n_devices)] == [4, 6, 5, 7]
+    assert mm.TileAssignmentDevices(out) == [4, 6, 5, 7]
+    o = so.to_mpmd_sharding(2, _oracle_op2({"type": "OTHER", "tile_dims": [2, 2], "tile_assignment_devices": [0, 2, 1, 3]}),
+                            (4, 4), (0, 8))
+    assert o.tile_assignment_devices == [4, 6, 5, 7]
+    with pytest.raises(mm.MmrError):
+        mm.ToMpmdSharding(2, mm.op_sharding("OTHER", [2, 1], tile_assignment_devices=[0, 5]), (4, 2), (0, 8))
