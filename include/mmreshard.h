@@ -132,6 +132,10 @@ int mmr_needs_reshard(int64_t operand_dev_start, int64_t operand_dev_count, int6
                       int64_t dev_count, const mmr_op_sharding* operand_sharding,
                       const mmr_op_sharding* sharding, int32_t* out);
 
+/* CreateDeviceList(tile_assignment), mpmd_utils.cc:151-175: the contiguous device range a sharding covers; an explicit
+ * list that is not consecutive ascending ids is MMR_UNSUPPORTED, as in the reference. */
+int mmr_device_list_of_sharding(const mmr_op_sharding* s, int64_t* dev_start, int64_t* dev_count);
+
 /* ToMpmdSharding, mpmd_partition.cc:128-166: a sharding written relative to a task's devices (ids 0..n-1, as it
  * stands inside the task's module) -> the sharding over global device ids.  rank = tensor rank.  An explicit
  * device list or a single device is written to devices_out (capacity entries) and out points at it. */

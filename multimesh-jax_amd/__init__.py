@@ -7,7 +7,7 @@ the reference's names for the path.
 from . import _binding
 from ._binding import LIB_PATH, MmrError, load  # noqa: F401
 from .api import (  # noqa: F401
-    CanonicalizeSharding, ComputeGlobalIndex, ComputeIndexSet, LogicalShardingToOpSharding, LogicalToPhysicalSharding,
+    CanonicalizeSharding, ComputeGlobalIndex, ComputeIndexSet, DeviceListOfSharding, LogicalShardingToOpSharding, LogicalToPhysicalSharding,
     MeshEquivalentSharding, NeedsReshard, Plan, ReshardContext, StoreHandle, TileAssignmentDevices, ToMpmdSharding,
     XlaShapeToZukuShape, describe, device_of_tile, itemsize, op_sharding, partition_spec_to_sharded_shape, shard_bytes,
     shard_extents,

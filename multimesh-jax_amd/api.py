@@ -181,6 +181,13 @@ def NeedsReshard(operand_devices: Tuple[int, int], devices: Tuple[int, int], ope
     return bool(out.value)
 
 
+def DeviceListOfSharding(sharding: B.OpSharding) -> Tuple[int, int]:
+    """(start, count) of the contiguous device range a sharding covers (mpmd_utils.cc:151-175)."""
+    start, count = C.c_int64(), C.c_int64()
+    B.check(B.load().mmr_device_list_of_sharding(C.byref(sharding), C.byref(start), C.byref(count)))
+    return start.value, count.value
+
+
 def ToMpmdSharding(rank: int, sharding: B.OpSharding, task_devices: Tuple[int, int],
                    global_devices: Tuple[int, int]) -> B.OpSharding:
     """A sharding written relative to a task's devices -> the sharding over global device ids

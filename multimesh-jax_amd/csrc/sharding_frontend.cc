@@ -417,6 +417,25 @@ int mmr_needs_reshard(int64_t operand_dev_start, int64_t operand_dev_count, int6
   return MMR_OK;
 }
 
+int mmr_device_list_of_sharding(const mmr_op_sharding* s, int64_t* dev_start, int64_t* dev_count) {
+  if (int rc = check_sharding(s)) return rc;
+  if (!dev_start || !dev_count) return fail(MMR_INVALID_ARGUMENT, "null output");
+  if (s->n_iota_dims > 0) {  // mpmd_utils.cc:158-165
+    int64_t n = 1;
+    for (int i = 0; i < s->n_iota_dims; ++i) n *= s->iota_reshape_dims[i];
+    *dev_start = s->iota_offset;
+    *dev_count = n;
+    return MMR_OK;
+  }
+  if (s->n_devices < 1 || !s->tile_assignment_devices) return fail(MMR_INVALID_ARGUMENT, "sharding names no devices");
+  for (int64_t i = 1; i < s->n_devices; ++i)  // :167-175
+    if (s->tile_assignment_devices[i] != s->tile_assignment_devices[i - 1] + 1)
+      return fail(MMR_UNSUPPORTED, "non-iota tile assignments not yet supported for DeviceList");
+  *dev_start = s->tile_assignment_devices[0];
+  *dev_count = s->n_devices;
+  return MMR_OK;
+}
+
 int mmr_to_mpmd_sharding(int32_t rank, const mmr_op_sharding* sharding, int64_t task_dev_start, int64_t task_dev_count,
                          int64_t global_dev_start, int64_t global_dev_count, mmr_op_sharding* out, int64_t* devices_out,
                          int64_t devices_capacity) {

@@ -331,3 +331,15 @@ def test_to_mpmd_sharding_special_cases():
     assert o.tile_assignment_devices == [4, 6, 5, 7]
     with pytest.raises(mm.MmrError):
         mm.ToMpmdSharding(2, mm.op_sharding("OTHER", [2, 1], tile_assignment_devices=[0, 5]), (4, 2), (0, 8))
+
+
+def test_device_list_of_a_sharding():
+    """CreateDeviceList (mpmd_utils.cc:151-175): an iota assignment covers [offset, offset + product of its dims);
+    an explicit list must be consecutive ascending ids, anything else is unsupported as in the reference."""
+    assert mm.DeviceListOfSharding(mm.op_sharding("OTHER", [2, 2], [2, 2], [1, 0], iota_offset=4)) == (4, 4)
+    assert mm.DeviceListOfSharding(mm.op_sharding("OTHER", [4, 1], tile_assignment_devices=[4, 5, 6, 7])) == (4, 4)
+    with pytest.raises(mm.MmrError, match="non-iota"):
+        mm.DeviceListOfSharding(mm.op_sharding("OTHER", [2, 2], tile_assignment_devices=[4, 6, 5, 7]))
+    # and through ToMpmdSharding: the rebased sharding of a task on devices 8-11 covers exactly those
+    rebased = mm.ToMpmdSharding(2, mm.op_sharding("OTHER", [4, 1], [4], [0]), (8, 4), (0, 12))
+    assert mm.DeviceListOfSharding(rebased) == (8, 4)
