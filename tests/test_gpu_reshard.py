@@ -557,3 +557,38 @@ def test_device_resident_shards_assemble_through_the_copy_kernel(ctx):
     say("device-to-device AssembleShards of %d MiB: %.1f us, %.0f GB/s (read + write)" % (n >> 20, ms * 1e3, 2 * n / ms / 1e6))
     for s in (src, dst):
         ctx.Free(s)
+
+
+def test_offsets_beyond_four_gigabytes(ctx):
+    """A 5 GiB shard buffer: chunk offsets, row strides and the flat copy's vector index need 64 bits.  One device
+    holding [rows, 4096] bytes -> two devices, rows split, the second stored column-major is left out on purpose
+    (plain copies only); bit-exact against NumPy slices of the same buffer."""
+    rows, cols = 5 * (1 << 30) // 4096 + 3, 4096
+    shape_src = mm.sharded_shape("U8", [(rows, 1, 0), (cols, 1, 1)], 0, 1)
+    shape_dst = mm.sharded_shape("U8", [(rows, 2, 0), (cols, 1, 1)], 1, 2)
+    rng = np.random.Generator(np.random.PCG64(4))
+    block = rng.integers(0, 256, size=(1 << 26), dtype=np.uint8)
+    data = np.empty(rows * cols, dtype=np.uint8)
+    for off in range(0, data.size, block.size):  # cheap, but different in every 64 MiB block
+        n = min(block.size, data.size - off)
+        np.add(block[:n], np.uint8((off >> 26) * 37 & 0xFF), out=data[off:off + n])
+    say("5 GiB shard: assembling")
+    src = ctx.CreateStore(shape_src, name="big.src")
+    ctx.AssembleShards(shape_src, 0, data, existing_store=src)
+    dst = ctx.CreateStore(shape_dst, name="big.dst")
+    say("5 GiB shard: resharding")
+    ctx.Reshard(src, dst)
+    ctx.Sync()
+    half = (rows + 1) // 2
+    for k, dev in enumerate(dst.devices):
+        got = ctx.ReadShard(dst, dev)
+        lo, hi = k * half, min((k + 1) * half, rows)
+        assert got[:(hi - lo) * cols].tobytes() == data[lo * cols:hi * cols].tobytes(), dev
+        assert not got[(hi - lo) * cols:].any()  # the pad row of the short tile is zero
+    # device-to-device assemble of the whole 5 GiB shard through the flat copy kernel
+    copy = ctx.CreateStore(shape_src, name="big.copy")
+    ctx.AssembleShards(shape_src, 0, ctx.SliceLocalShard(0, src), existing_store=copy, size=rows * cols)
+    ctx.Sync()
+    assert ctx.ReadShard(copy, 0).tobytes() == data.tobytes()
+    for s in (src, dst, copy):
+        ctx.Free(s)
