@@ -192,7 +192,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "u128" if res["kernel"] == "mmr_copy16_kernel" else "u8",
+        "dtype": "u8",  # pure byte movement (bf16 payload never interpreted), 16-byte vector accesses
         "data": "synthetic",
         "config": {
             "workload": "configuration %d of BASELINE.json: %s" % (
