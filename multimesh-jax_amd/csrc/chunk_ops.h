@@ -12,7 +12,7 @@
 //   static V16 load16(cptr), load16u(cptr);       16-byte load, aligned / any alignment
 //   static void store16(ptr, V16);                16-byte aligned store
 //   static T loadu<T>(cptr); static void storeu<T>(ptr, T);   1/2/4/8-byte, any alignment
-//   static uintptr_t addr(ptr);                   numeric address (for alignment math)
+//   static uintptr_t addr(ptr), caddr(cptr);      numeric address (for alignment math)
 #ifndef MMR_CSRC_CHUNK_OPS_H_
 #define MMR_CSRC_CHUNK_OPS_H_
 
@@ -128,13 +128,16 @@ MMR_HD void copy16_chunk(const mmr_copy_chunk& c, typename M::cptr src, typename
 // ---------------------------------------------------------------------------
 // Generic copy: n1 rows of any width at any byte alignment on either side
 // (the planner emits generic chunks with n2 == 1).  Each row is cut at the
-// 16-byte boundaries of its DESTINATION: a lane owns one aligned 16-byte slot,
-// loads the matching source bytes with one unaligned 16-byte load and writes
-// one 16-byte store.  A slot cut off by a row end (the first and the last slot
-// of a row, in general) slides inwards until it lies inside the row: it still
-// moves 16 bytes, now at an unaligned destination address, and overlaps its
-// neighbour, which writes the same values to the shared bytes.  So every lane
-// runs the same two instructions and no access ever leaves its row.  Rows
+// 16-byte boundaries of its SOURCE (of its destination when the chunk fills):
+// a lane owns one aligned 16-byte slot, loads it with one 16-byte load and
+// writes the matching destination bytes with one 16-byte store at whatever
+// alignment they have - measured on MI355X, a misaligned store costs less than
+// a misaligned load (2-3 % of the kernel time on byte-misaligned rows).  A slot
+// cut off by a row end (the first and the last slot of a row, in general)
+// slides inwards until it lies inside the row: it still moves 16 bytes, now
+// unaligned on both sides, and overlaps its neighbour, which writes the same
+// values to the shared bytes.  So every lane runs the same two instructions
+// and no access ever leaves its row.  Rows
 // narrower than 16 bytes have no room to slide: their 1..15 bytes move as
 // 8/4/2/1-byte pieces (binary decomposition of the length), carried in one V16:
 // .x/.y the 8-byte piece, .z the 4-byte piece, .w the 2-byte piece (low half)
@@ -171,7 +174,7 @@ MMR_HD void generic_load(const mmr_copy_chunk& c, typename M::cptr src, typename
   typename M::ptr drow = dst + row * c.d1;
   typename M::cptr srow = src + row * c.s1;
   const int32_t w = static_cast<int32_t>(c.w);
-  const int32_t mis = static_cast<int32_t>(M::addr(drow) & 15u);
+  const int32_t mis = static_cast<int32_t>((fill ? M::addr(drow) : M::caddr(srow)) & 15u);
   const int32_t rel = static_cast<int32_t>(slot << 4) - mis;  // row-relative byte where this aligned slot starts
   if constexpr (WIDE) {
     if (rel >= w) {
@@ -194,7 +197,7 @@ MMR_HD void generic_load(const mmr_copy_chunk& c, typename M::cptr src, typename
 template <class M, bool WIDE>
 MMR_HD void generic_store(typename M::ptr dpos, int32_t len, V16 v) {
   if constexpr (WIDE) {
-    if (len != 0) M::template storeu<V16>(dpos, v);  // aligned except for the slots that slid inwards
+    if (len != 0) M::template storeu<V16>(dpos, v);
   } else {
     if (len > 0) store_ragged<M>(dpos, static_cast<uint32_t>(len), v);
   }

@@ -70,6 +70,7 @@ struct DeviceMem {
     else st<T, 1>(p, v);
   }
   static __device__ __forceinline__ uintptr_t addr(ptr p) { return reinterpret_cast<uintptr_t>(p); }
+  static __device__ __forceinline__ uintptr_t caddr(cptr p) { return reinterpret_cast<uintptr_t>(p); }
 };
 
 __device__ __forceinline__ gchar* slot_base(void* const* __restrict__ ptrs, uint32_t slot, uint64_t off) {

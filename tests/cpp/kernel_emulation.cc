@@ -73,6 +73,7 @@ struct HostMem {
   template <typename T>
   static void storeu(ptr p, T v) { put<T>(p, v, 1, "out-of-bounds store"); }
   static uintptr_t addr(ptr p) { return reinterpret_cast<uintptr_t>(p); }
+  static uintptr_t caddr(cptr p) { return reinterpret_cast<uintptr_t>(p); }
 };
 
 template <typename T>
