@@ -109,7 +109,9 @@ def measure(ctx, mm, workloads, args, config, with_parity=True):
     ctx.Sync()
     wall_s = time.perf_counter() - t0
 
-    plan = ctx.plan_stats(sets[0][0][0], sets[0][1][0]) if len(arrays) == 1 else None
+    batched = len(arrays) > 1 and not getattr(args, "unbatched", False)
+    plan = (ctx.plan_stats(sets[0][0][0], sets[0][1][0]) if len(arrays) == 1 else
+            ctx.batch_plan_stats(sets[0][0], sets[0][1]) if batched else None)
     # cold plan construction (host only, excluded from the steady-state figure: plans are cached per descriptor pair)
     from helpers import lib_shape
     src_shapes = [lib_shape(a["type"], a["src"]) for a in arrays]

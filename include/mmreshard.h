@@ -364,6 +364,9 @@ typedef struct {
 int mmr_context_get_stats(mmr_context* ctx, mmr_context_stats* out);
 /* Stats of the cached plan of a store pair (builds it if needed). */
 int mmr_reshard_plan_stats(mmr_context* ctx, mmr_store* src, mmr_store* dst, mmr_plan_stats* out);
+/* The same for the plan of a batch (the arrays in the order mmr_reshard_batch was or will be given them). */
+int mmr_reshard_batch_plan_stats(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int32_t n,
+                                 mmr_plan_stats* out);
 
 #ifdef __cplusplus
 }

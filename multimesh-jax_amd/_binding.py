@@ -158,6 +158,7 @@ PROTOTYPES = {
     "mmr_timer_stop": (C.c_int, [VP, P(C.c_float)]),
     "mmr_context_get_stats": (C.c_int, [VP, P(ContextStats)]),
     "mmr_reshard_plan_stats": (C.c_int, [VP, VP, VP, P(PlanStats)]),
+    "mmr_reshard_batch_plan_stats": (C.c_int, [VP, P(VP), P(VP), I32, P(PlanStats)]),
 }
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libmmreshard.so")

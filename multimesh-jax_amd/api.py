@@ -475,3 +475,14 @@ class ReshardContext:
         st = B.PlanStats()
         B.check(self._lib.mmr_reshard_plan_stats(self._h, src._h, dst._h, C.byref(st)))
         return st.as_dict()
+
+    def batch_plan_stats(self, srcs: Sequence[StoreHandle], dsts: Sequence[StoreHandle]) -> dict:
+        """Stats of the plan a ReshardBatch of these stores uses (table order chosen on first use included)."""
+        n = len(srcs)
+        if n == 0 or n != len(dsts):
+            raise ValueError("as many destinations as sources, at least one")
+        sa = (C.c_void_p * n)(*[s._h for s in srcs])
+        da = (C.c_void_p * n)(*[d._h for d in dsts])
+        st = B.PlanStats()
+        B.check(self._lib.mmr_reshard_batch_plan_stats(self._h, sa, da, n, C.byref(st)))
+        return st.as_dict()

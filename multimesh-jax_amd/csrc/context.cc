@@ -745,16 +745,26 @@ int mmr_context_get_stats(mmr_context* ctx, mmr_context_stats* out) {
   return MMR_OK;
 }
 
-int mmr_reshard_plan_stats(mmr_context* ctx, mmr_store* src, mmr_store* dst, mmr_plan_stats* out) {
-  if (!ctx || !out) return fail(MMR_INVALID_ARGUMENT, "null argument");
+int mmr_reshard_batch_plan_stats(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int32_t n,
+                                 mmr_plan_stats* out) {
+  if (!ctx || !out || n <= 0 || !srcs || !dsts) return fail(MMR_INVALID_ARGUMENT, "bad arguments");
   std::lock_guard<std::mutex> lock(ctx->mu);
-  if (int rc = check_store(ctx, src, "source")) return rc;
-  if (int rc = check_store(ctx, dst, "destination")) return rc;
+  std::vector<mmr_sharded_shape> s(static_cast<size_t>(n)), d(static_cast<size_t>(n));
+  for (int a = 0; a < n; ++a) {
+    if (int rc = check_store(ctx, srcs[a], "source")) return rc;
+    if (int rc = check_store(ctx, dsts[a], "destination")) return rc;
+    s[a] = srcs[a]->shape;
+    d[a] = dsts[a]->shape;
+  }
   if (int rc = use_device(ctx)) return rc;
   DevicePlan* dp = nullptr;
-  if (int rc = get_plan(ctx, {src->shape}, {dst->shape}, &dp)) return rc;
+  if (int rc = get_plan(ctx, s, d, &dp)) return rc;
   *out = dp->plan.stats;
   return MMR_OK;
+}
+
+int mmr_reshard_plan_stats(mmr_context* ctx, mmr_store* src, mmr_store* dst, mmr_plan_stats* out) {
+  return mmr_reshard_batch_plan_stats(ctx, &src, &dst, 1, out);
 }
 
 }  // extern "C"

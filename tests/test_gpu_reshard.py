@@ -160,7 +160,18 @@ def test_random_batch_mixed_kernels(ctx):
         gs.append(rng.integers(0, 256, size=int(np.prod(a["shape"])) * item, dtype=np.uint8).view(
             ro.raw_dtype(a["type"])).reshape(a["shape"]))
     say("random batch of 25 arrays")
-    _compare(arrays, gs, gpu_reshard(ctx, arrays, gs, batch=True))
+    outs, srcs, dsts = gpu_reshard(ctx, arrays, gs, batch=True, keep=True)
+    _compare(arrays, gs, outs)
+    # the batch has one plan of its own; its stats count every array and every kernel class of the batch
+    built = ctx.stats["plans_built"]
+    st = ctx.batch_plan_stats(srcs, dsts)
+    assert ctx.stats["plans_built"] == built, "the stats call found the batch's cached plan"
+    assert st["n_arrays"] == 25
+    # every element is written once per destination replica
+    assert st["bytes_moved"] == sum(g.nbytes * (a["dst"]["dims"][-1][1] if len(a["dst"]["dims"]) > g.ndim else 1)
+                                    for a, g in zip(arrays, gs))
+    for s in srcs + dsts:
+        ctx.Free(s)
 
 
 @pytest.mark.parametrize("type_", ["U8", "BF16", "F32", "F64", "C128"])
