@@ -28,6 +28,8 @@ struct BoxDim {
 
 int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+constexpr int64_t kGenericMaxPairs = 768;  // (row, slot) pairs of one generic chunk
+
 class Builder {
  public:
   Builder(mmr_plan* plan, uint32_t chunk_bytes, uint32_t generic_chunk_bytes, bool force_generic)
@@ -152,7 +154,15 @@ class Builder {
       });
       return;
     }
-    const int64_t rows = std::max<int64_t>(1, cb / w);
+    int64_t rows = std::max<int64_t>(1, cb / w);
+    if (!aligned) {
+      // The generic kernel spends one lane per (row, 16-byte slot) pair whatever the row holds: a chunk of very
+      // narrow rows sized by bytes alone (the one-byte pad column of a short edge tile: 5,632 rows) keeps its
+      // workgroup busy long after its neighbours have finished and becomes the tail of the launch.  Bound the
+      // pairs per chunk (3 per lane of a 256-lane workgroup) as well as the bytes.
+      const int64_t slots = (w + 15) / 16 + 1;
+      rows = std::max<int64_t>(1, std::min(rows, kGenericMaxPairs / slots));
+    }
     int i1 = pick_row_dim(outer, -1);
     if (i1 < 0) {
       emit_copy(src_slot, dst_slot, so, dof, w, 1, 1, 0, 0, 0, 0, fill);

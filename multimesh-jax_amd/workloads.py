@@ -112,6 +112,9 @@ def config(index: int, scale: int = 1) -> List[dict]:
     if index == 16:  # probe: configuration 10's split with 16-byte aligned pieces (816 / 544 / 272-byte rows)
         b = (88064 // s, 4080)
         return [_array("probe_u8_aligned", "U8", b, _side(b, (1, 3), 0), _side(b, (1, 5), 3), 6, "raw")]
+    if index == 17:  # probe: byte-misaligned source rows (1387 bytes), destination rows of 832 bytes = 13 x 64
+        b = (88064 // s, 4160)
+        return [_array("probe_u8_dst64", "U8", b, _side(b, (1, 3), 0), _side(b, (1, 5), 3), 6, "raw")]
     if index == 7:  # probe: 4-byte elements, uneven 3-way -> 5-way (dword-aligned, not 16-byte-aligned runs)
         b = (11008 // s, 1025)
         return [_array("probe_s32", "S32", b, _side(b, (1, 3), 0), _side(b, (1, 5), 3), 7, "raw")]
