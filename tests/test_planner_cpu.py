@@ -169,3 +169,23 @@ def test_plan_rejects_mismatched_pairs():
         bad.dtype = 55
         mm.Plan(bad, bad)
     assert e.value.status_name == "UNSUPPORTED"
+
+
+def test_generic_chunks_are_bounded_in_lane_work_as_well_as_in_bytes():
+    """The generic kernel spends one lane per (row, 16-byte slot) pair: the one-byte pad
+    column of configuration 5's last tile must not come out as chunks of thousands of
+    rows (each would keep one workgroup busy long after the rest of the launch)."""
+    arrays = workloads.config(5)
+    plan = mm.Plan([lib_shape(a["type"], a["src"]) for a in arrays],
+                   [lib_shape(a["type"], a["dst"]) for a in arrays])
+    g = plan.copy_chunks(1)
+    assert len(g) > 0 and len(plan.copy_chunks(0)) == 0
+    slots = (g["w"].astype(np.int64) + 15) // 16 + 1
+    pairs = g["n1"].astype(np.int64) * g["n2"] * slots
+    assert pairs.max() <= 768
+    fills = g[g["src_slot"] == 0xFFFFFFFF]
+    assert plan.stats["n_fill_chunks"] == len(fills)
+    fp8_pad = fills[fills["w"] == 1]  # 11008 rows x 1 byte after the 819 valid bytes of the last tile
+    assert int(fp8_pad["n1"].sum()) == 11008 and fp8_pad["n1"].max() <= 384
+    # whole rows of 820 bytes come eight to a chunk (7 KiB)
+    assert int(g[g["w"] == 820]["n1"].max()) == 8
