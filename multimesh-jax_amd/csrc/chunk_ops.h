@@ -265,19 +265,32 @@ MMR_HD void generic_chunk(const mmr_copy_chunk& c, typename M::cptr src, typenam
 // kEX x kEY sub-tile each (kWX x kWY waves; for 1-byte elements all four waves
 // share one sub-tile).
 //
-// Vector path (tile 16-byte aligned on both sides, extents multiples of the
-// vector width): every wave works alone, on its own slice of LDS, so the only
-// synchronisation is between the lanes of a wave (the caller puts a wave-level
-// fence between the two phases; a workgroup barrier where waves share a
-// sub-tile).  Every global
-// access is a 16-byte vector and every LDS access at least a dword.  A lane
-// loads the same vector of kPack = 4 / itemsize adjacent source rows (one row
-// for elements of 4 bytes and more), so for each of the vector's x it holds
-// kPack consecutive y: one dword (or one element of 8 / 16 bytes), written to
-// row x of an LDS tile laid out [x][y] without padding.  In the second phase a
-// lane reads one 16-byte group of an LDS row = consecutive y of one x and
-// stores it to destination row x.  All global loads of a lane are issued before
-// its first LDS write.
+// Every wave works alone, on its own sub-tile and its own slice of LDS, so the
+// only synchronisation is between the lanes of a wave (the caller puts a
+// wave-level fence between the two phases; a workgroup barrier where waves
+// share a sub-tile).  What a wave does with its sub-tile depends on the part of
+// it that lies inside the tile (snx x sny elements):
+//
+// Vector path (chunk 16-byte aligned on both sides, snx and sny multiples of
+// the vector width): every global access is an aligned 16-byte vector and every
+// LDS access at least a dword.  A lane loads the same vector of kPack =
+// 4 / itemsize adjacent source rows (one row for elements of 4 bytes and more),
+// so for each of the vector's x it holds kPack consecutive y: one dword (or one
+// element of 8 / 16 bytes), written to row x of an LDS tile laid out [x][y]
+// without padding.  In the second phase a lane reads one 16-byte group of an
+// LDS row = consecutive y of one x and stores it to destination row x.  All
+// global loads of a lane are issued before its first LDS write.
+//
+// General path (any alignment, snx and sny at least one vector): the same with
+// unaligned 16-byte global accesses.  A vector cut off by the edge of the tile
+// slides inwards until it ends at the edge (it overlaps its neighbour, which
+// moves the same values); a packed source row beyond the edge is replaced by
+// the last row inside (its LDS cells are never read).  A destination vector
+// that slid is gathered from LDS element by element.  No access leaves the
+// tile.
+//
+// Element path (a sub-tile thinner than one vector): one element per lane and
+// step, same LDS layout.
 //
 // LDS banks: rows are a multiple of 128 bytes apart, so the 16-byte groups of a
 // row are permuted by XOR with a function of x whose low three bits differ
@@ -285,11 +298,6 @@ MMR_HD void generic_chunk(const mmr_copy_chunk& c, typename M::cptr src, typenam
 // between any 8 consecutive x): the dword writes of 32 lanes then fall into 32
 // different banks.  Reads are conflict-free by construction (8 consecutive
 // lanes read the 8 groups of one 128-byte row segment).
-//
-// Element path (anything else, e.g. ragged edge tiles): the whole workgroup
-// walks the sub-tiles one after the other, one element per lane, LDS laid out
-// [y][x] with pitch kEX + 1; the caller puts a workgroup barrier after each
-// phase.
 // ---------------------------------------------------------------------------
 template <int ITEM>
 struct TransposeTile {
@@ -306,19 +314,17 @@ struct TransposeTile {
   static constexpr int kTileX = kEX * kWX, kTileY = kEY * kWY;
   static constexpr int kVec = 16 / ITEM;                     // elements per 16-byte vector
   static constexpr int kPack = ITEM >= 4 ? 1 : 4 / ITEM;     // source rows a lane packs into one LDS word
-  static constexpr int kRowBytes = kEY * ITEM;               // vector path: bytes per LDS row (no padding)
+  static constexpr int kRowBytes = kEY * ITEM;               // bytes per LDS row (no padding)
   static constexpr int kSrcVecs = kEX / kVec;                // 16-byte groups per source row of a sub-tile
   static constexpr int kDstVecs = kEY / kVec;                // 16-byte groups per destination row of a sub-tile
   static constexpr int kRowPacks = kEY / kPack;              // packed source-row groups per sub-tile
-  static constexpr int kWaveLdsBytes = kEX * kEY * ITEM;     // vector path: one wave's slice
-  static constexpr int kPitch1 = kEX + 1;                    // element path, elements
-  static constexpr int kLdsBytes =
-      kWaveLdsBytes * kWaves > kEY * kPitch1 * ITEM ? kWaveLdsBytes * kWaves : kEY * kPitch1 * ITEM;
+  static constexpr int kWaveLdsBytes = kEX * kEY * ITEM;     // one sub-tile's slice
+  static constexpr int kLdsBytes = kWaveLdsBytes * kWaves;
   static_assert(kSrcVecs % 8 == 0 && kDstVecs % 8 == 0, "sub-tile rows must be whole 128-byte lines");
   static_assert(kSrcVecs * kRowPacks % kGroupThreads == 0 && kEX * kDstVecs % kGroupThreads == 0,
                 "sub-tile must divide over its threads");
 };
-constexpr int kTransposeLdsBytes = 32 * 1024 + 1024;  // at least the largest TransposeTile<>::kLdsBytes
+constexpr int kTransposeLdsBytes = 32 * 1024;  // the largest TransposeTile<>::kLdsBytes
 
 // Workgroup tile extents in elements for an element width (the planner cuts boxes into these).
 inline void transpose_tile_extent(uint32_t itemsize, uint32_t* tile_x, uint32_t* tile_y) {
@@ -331,11 +337,21 @@ inline void transpose_tile_extent(uint32_t itemsize, uint32_t* tile_x, uint32_t*
   }
 }
 
-MMR_HD bool transpose_is_vector(const mmr_transpose_chunk& c) {
-  const uint32_t vec = 16u / c.itemsize;
+// What a wave does with its sub-tile (uniform over the threads that share the sub-tile).
+enum TransposeMode { kTransposeNothing = 0, kTransposeVector = 1, kTransposeGeneral = 2, kTransposeElement = 3 };
+
+MMR_HD bool transpose_is_aligned(const mmr_transpose_chunk& c) {
   const uint64_t bits = c.src_off | c.dst_off | static_cast<uint64_t>(c.src_ystride) | static_cast<uint64_t>(c.dst_xstride) |
                         static_cast<uint64_t>(c.src_bstride) | static_cast<uint64_t>(c.dst_bstride);
-  return (bits & 15u) == 0 && c.nx % vec == 0 && c.ny % vec == 0;
+  return (bits & 15u) == 0;
+}
+
+// A chunk whose every sub-tile takes the vector path (or lies outside the tile).  Such chunks run through a kernel
+// that holds nothing but the vector path: with the general and the element path compiled in, the kernel needs twice
+// the registers and runs at half the occupancy.  The planner keeps the two kinds apart in the table.
+MMR_HD bool transpose_is_vector(const mmr_transpose_chunk& c) {
+  const uint32_t vec = 16u / c.itemsize;
+  return transpose_is_aligned(c) && c.nx % vec == 0 && c.ny % vec == 0;
 }
 
 // XOR applied to the 16-byte group index of LDS row x.
@@ -378,7 +394,55 @@ MMR_HD void transpose_subtile(uint32_t wave, uint32_t* x0, uint32_t* y0) {
   *y0 = (wave / G::kWX) * G::kEY;
 }
 
-// Vector path, phase 1: global -> registers -> this wave's LDS slice.  tid = thread of the workgroup.
+// The part of sub-tile `wave` that lies inside the tile, and what to do with it.
+template <int ITEM>
+MMR_HD TransposeMode transpose_mode(const mmr_transpose_chunk& c, uint32_t wave, uint32_t* x0, uint32_t* y0, uint32_t* snx,
+                                    uint32_t* sny) {
+  typedef TransposeTile<ITEM> G;
+  transpose_subtile<ITEM>(wave, x0, y0);
+  *snx = c.nx > *x0 ? (c.nx - *x0 < static_cast<uint32_t>(G::kEX) ? c.nx - *x0 : static_cast<uint32_t>(G::kEX)) : 0u;
+  *sny = c.ny > *y0 ? (c.ny - *y0 < static_cast<uint32_t>(G::kEY) ? c.ny - *y0 : static_cast<uint32_t>(G::kEY)) : 0u;
+  if (*snx == 0 || *sny == 0) return kTransposeNothing;
+  if (*snx % G::kVec == 0 && *sny % G::kVec == 0 && transpose_is_aligned(c)) return kTransposeVector;
+  if (*snx >= static_cast<uint32_t>(G::kVec) && *sny >= static_cast<uint32_t>(G::kVec)) return kTransposeGeneral;
+  return kTransposeElement;
+}
+
+// LDS address of element (x, y) of a sub-tile slice: row x, 16-byte groups of the row permuted.
+template <int ITEM>
+MMR_HD uint32_t transpose_lds_offset(uint32_t x, uint32_t y) {
+  const uint32_t ybyte = y * static_cast<uint32_t>(ITEM);
+  return x * TransposeTile<ITEM>::kRowBytes + (((ybyte >> 4) ^ transpose_swizzle<ITEM>(x)) << 4) + (ybyte & 15u);
+}
+
+template <typename T>
+MMR_HD void set_element(V16* v, int i, T e) {
+  // i is a compile-time constant after unrolling; *v starts as zero
+  if constexpr (sizeof(T) == 16) {
+    *v = e;
+  } else if constexpr (sizeof(T) == 8) {
+    if (i == 0) {
+      v->x = static_cast<uint32_t>(e);
+      v->y = static_cast<uint32_t>(e >> 32);
+    } else {
+      v->z = static_cast<uint32_t>(e);
+      v->w = static_cast<uint32_t>(e >> 32);
+    }
+  } else {
+    constexpr int per = 4 / static_cast<int>(sizeof(T));
+    const uint32_t bits = static_cast<uint32_t>(e) << (8 * static_cast<int>(sizeof(T)) * (i % per));
+    if (i / per == 0) v->x |= bits;
+    else if (i / per == 1) v->y |= bits;
+    else if (i / per == 2) v->z |= bits;
+    else v->w |= bits;
+  }
+}
+
+// Vector path, phase 1: global -> registers -> this wave's LDS slice.  tid = thread of the workgroup.  The
+// sub-tile must hold at least one vector (the callers skip sub-tiles outside the tile).  No lane is predicated: a
+// task that falls outside the tile loads the sub-tile's first vector again and parks it in LDS cells that nobody
+// reads (every task's cells lie inside the wave's slice), so the loads are straight-line code and all of them are
+// in flight before the first LDS write.
 template <class M, typename T>
 MMR_HD void transpose_load_vec(const mmr_transpose_chunk& c, typename M::cptr src, uint32_t b, T* lds, uint32_t tid) {
   typedef TransposeTile<sizeof(T)> G;
@@ -393,31 +457,29 @@ MMR_HD void transpose_load_vec(const mmr_transpose_chunk& c, typename M::cptr sr
   for (int k = 0; k < kTasks; ++k) {
     uint32_t yg, xv;
     transpose_task(lane + k * G::kGroupThreads, G::kRowPacks, &yg, &xv);
-    if (y0 + yg * G::kPack < c.ny && x0 + xv * G::kVec < c.nx) {
+    const bool inside = y0 + yg * G::kPack < c.ny && x0 + xv * G::kVec < c.nx;
+    const uint32_t yl = inside ? yg * G::kPack : 0u, xl = inside ? xv : 0u;
 #pragma unroll
-      for (int p = 0; p < G::kPack; ++p)
-        v[k][p] = M::load16(s + ((yg * G::kPack + p) * c.src_ystride + static_cast<int64_t>(xv) * 16));
-    }
+    for (int p = 0; p < G::kPack; ++p)
+      v[k][p] = M::load16(s + ((yl + p) * c.src_ystride + static_cast<int64_t>(xl) * 16));
   }
 #pragma unroll
   for (int k = 0; k < kTasks; ++k) {
     uint32_t yg, xv;
     transpose_task(lane + k * G::kGroupThreads, G::kRowPacks, &yg, &xv);
-    if (y0 + yg * G::kPack < c.ny && x0 + xv * G::kVec < c.nx) {
-      const uint32_t ybyte = yg * G::kPack * static_cast<uint32_t>(sizeof(T));  // byte of y within LDS row x
+    const uint32_t ybyte = yg * G::kPack * static_cast<uint32_t>(sizeof(T));  // byte of y within LDS row x
 #pragma unroll
-      for (int i = 0; i < G::kVec; ++i) {
-        const uint32_t x = xv * G::kVec + i;
-        uint8_t* at = tile + x * G::kRowBytes + (((ybyte >> 4) ^ transpose_swizzle<sizeof(T)>(x)) << 4) + (ybyte & 15u);
-        if constexpr (sizeof(T) >= 4) {
-          *reinterpret_cast<T*>(at) = element_of<T>(v[k][0], i);
-        } else {
-          uint32_t word = 0;
+    for (int i = 0; i < G::kVec; ++i) {
+      const uint32_t x = xv * G::kVec + i;
+      uint8_t* at = tile + x * G::kRowBytes + (((ybyte >> 4) ^ transpose_swizzle<sizeof(T)>(x)) << 4) + (ybyte & 15u);
+      if constexpr (sizeof(T) >= 4) {
+        *reinterpret_cast<T*>(at) = element_of<T>(v[k][0], i);
+      } else {
+        uint32_t word = 0;
 #pragma unroll
-          for (int p = 0; p < G::kPack; ++p)
-            word |= static_cast<uint32_t>(element_of<T>(v[k][p], i)) << (8 * static_cast<int>(sizeof(T)) * p);
-          *reinterpret_cast<uint32_t*>(at) = word;
-        }
+        for (int p = 0; p < G::kPack; ++p)
+          word |= static_cast<uint32_t>(element_of<T>(v[k][p], i)) << (8 * static_cast<int>(sizeof(T)) * p);
+        *reinterpret_cast<uint32_t*>(at) = word;
       }
     }
   }
@@ -449,36 +511,245 @@ MMR_HD void transpose_store_vec(const mmr_transpose_chunk& c, typename M::ptr ds
   }
 }
 
-// Element path: sub-tile `sub` of the workgroup tile, all threads of the workgroup.
+// General path, phase 1.  (x0, y0) origin and snx x sny valid extent of this wave's sub-tile (at least one vector
+// each way).  No lane is predicated here either: a vector beyond the edge becomes the last vector inside, a row
+// beyond the edge the last row inside; what such a task writes to LDS either repeats what the rightful task writes
+// to the same cells or lands in cells of rows y >= sny, which nobody reads.
 template <class M, typename T>
-MMR_HD void transpose_load(const mmr_transpose_chunk& c, typename M::cptr src, uint32_t b, uint32_t sub, T* lds, uint32_t tid) {
+MMR_HD void transpose_load_general(const mmr_transpose_chunk& c, typename M::cptr src, uint32_t b, T* lds, uint32_t tid,
+                                   uint32_t x0, uint32_t y0, uint32_t snx, uint32_t sny) {
   typedef TransposeTile<sizeof(T)> G;
-  uint32_t x0, y0;
-  transpose_subtile<sizeof(T)>(sub, &x0, &y0);
-  if (x0 >= c.nx || y0 >= c.ny) return;
-  const uint32_t nx = c.nx - x0 < G::kEX ? c.nx - x0 : G::kEX, ny = c.ny - y0 < G::kEY ? c.ny - y0 : G::kEY;
+  constexpr int kTasks = G::kSrcVecs * G::kRowPacks / G::kGroupThreads;  // per lane
+  const uint32_t wave = tid / G::kGroupThreads, lane = tid % G::kGroupThreads;
   typename M::cptr s = src + (b * c.src_bstride + y0 * c.src_ystride + static_cast<int64_t>(x0) * static_cast<int64_t>(sizeof(T)));
-  const uint32_t n = nx * ny;
-  for (uint32_t i = tid; i < n; i += G::kThreads) {
-    const uint32_t y = i / nx, x = i - y * nx;
-    lds[y * G::kPitch1 + x] =
-        M::template loadu<T>(s + (y * c.src_ystride + static_cast<int64_t>(x) * static_cast<int64_t>(sizeof(T))));
+  uint8_t* tile = reinterpret_cast<uint8_t*>(lds) + wave * G::kWaveLdsBytes;
+  V16 v[kTasks][G::kPack];
+  uint32_t xs[kTasks];
+#pragma unroll
+  for (int k = 0; k < kTasks; ++k) {
+    uint32_t yg, xv;
+    transpose_task(lane + k * G::kGroupThreads, G::kRowPacks, &yg, &xv);
+    xs[k] = xv * G::kVec + G::kVec > snx ? snx - G::kVec : xv * G::kVec;  // slides inwards, overlapping its neighbour
+#pragma unroll
+    for (int p = 0; p < G::kPack; ++p) {
+      const uint32_t y = yg * G::kPack + p < sny ? yg * G::kPack + p : sny - 1;  // past the edge: the last row again
+      v[k][p] = M::load16u(s + (y * c.src_ystride + static_cast<int64_t>(xs[k]) * static_cast<int64_t>(sizeof(T))));
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < kTasks; ++k) {
+    uint32_t yg, xv;
+    transpose_task(lane + k * G::kGroupThreads, G::kRowPacks, &yg, &xv);
+#pragma unroll
+    for (int i = 0; i < G::kVec; ++i) {
+      uint8_t* at = tile + transpose_lds_offset<sizeof(T)>(xs[k] + i, yg * G::kPack);
+      if constexpr (sizeof(T) >= 4) {
+        *reinterpret_cast<T*>(at) = element_of<T>(v[k][0], i);
+      } else {
+        uint32_t word = 0;
+#pragma unroll
+        for (int p = 0; p < G::kPack; ++p)
+          word |= static_cast<uint32_t>(element_of<T>(v[k][p], i)) << (8 * static_cast<int>(sizeof(T)) * p);
+        *reinterpret_cast<uint32_t*>(at) = word;
+      }
+    }
+  }
+}
+
+// General path, phase 2.
+template <class M, typename T>
+MMR_HD void transpose_store_general(const mmr_transpose_chunk& c, typename M::ptr dst, uint32_t b, const T* lds, uint32_t tid,
+                                    uint32_t x0, uint32_t y0, uint32_t snx, uint32_t sny) {
+  typedef TransposeTile<sizeof(T)> G;
+  constexpr int kTasks = G::kEX * G::kDstVecs / G::kGroupThreads;  // per lane
+  const uint32_t wave = tid / G::kGroupThreads, lane = tid % G::kGroupThreads;
+  typename M::ptr d = dst + (b * c.dst_bstride + x0 * c.dst_xstride + static_cast<int64_t>(y0) * static_cast<int64_t>(sizeof(T)));
+  const uint8_t* tile = reinterpret_cast<const uint8_t*>(lds) + wave * G::kWaveLdsBytes;
+  V16 v[kTasks];
+  uint32_t ys[kTasks];
+#pragma unroll
+  for (int k = 0; k < kTasks; ++k) {
+    uint32_t x, yv;
+    transpose_task(lane + k * G::kGroupThreads, G::kEX, &x, &yv);
+    ys[k] = yv * G::kVec;
+    if (x < snx && ys[k] < sny) {
+      if (ys[k] + G::kVec <= sny) {
+        v[k] = *reinterpret_cast<const V16*>(tile + x * G::kRowBytes + ((yv ^ transpose_swizzle<sizeof(T)>(x)) << 4));
+      } else {  // cut off by the edge: slides inwards and is gathered element by element
+        ys[k] = sny - G::kVec;
+        v[k] = V16{0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < G::kVec; ++i)
+          set_element<T>(&v[k], i, *reinterpret_cast<const T*>(tile + transpose_lds_offset<sizeof(T)>(x, ys[k] + i)));
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < kTasks; ++k) {
+    uint32_t x, yv;
+    transpose_task(lane + k * G::kGroupThreads, G::kEX, &x, &yv);
+    if (x < snx && yv * G::kVec < sny)
+      M::template storeu<V16>(d + (x * c.dst_xstride + static_cast<int64_t>(ys[k]) * static_cast<int64_t>(sizeof(T))), v[k]);
+  }
+}
+
+// Element path, both phases: a sub-tile thinner than one vector, at most kTransposeThin elements per lane.  All
+// loads of a lane are issued before its first LDS write; one division per phase, the (row, column) of a lane's
+// next element follows by a fixed step with a carry.
+constexpr int kTransposeThin = 8;
+
+template <class M, typename T>
+MMR_HD void transpose_load_element(const mmr_transpose_chunk& c, typename M::cptr src, uint32_t b, T* lds, uint32_t tid,
+                                   uint32_t x0, uint32_t y0, uint32_t snx, uint32_t sny) {
+  typedef TransposeTile<sizeof(T)> G;
+  static_assert((G::kEX > G::kEY ? G::kEX : G::kEY) * (G::kVec - 1) <= kTransposeThin * G::kGroupThreads,
+                "a thin sub-tile must fit the unrolled element path");
+  const uint32_t wave = tid / G::kGroupThreads, lane = tid % G::kGroupThreads;
+  typename M::cptr s = src + (b * c.src_bstride + y0 * c.src_ystride + static_cast<int64_t>(x0) * static_cast<int64_t>(sizeof(T)));
+  uint8_t* tile = reinterpret_cast<uint8_t*>(lds) + wave * G::kWaveLdsBytes;
+  const uint32_t n = snx * sny;
+  const uint32_t step_y = G::kGroupThreads / snx, step_x = G::kGroupThreads - step_y * snx;
+  uint32_t y = lane / snx, x = lane - y * snx;
+  T e[kTransposeThin];
+  uint32_t at[kTransposeThin];
+#pragma unroll
+  for (int k = 0; k < kTransposeThin; ++k) {
+    if (lane + k * G::kGroupThreads < n) {
+      e[k] = M::template loadu<T>(s + (y * c.src_ystride + static_cast<int64_t>(x) * static_cast<int64_t>(sizeof(T))));
+      at[k] = transpose_lds_offset<sizeof(T)>(x, y);
+    }
+    x += step_x;
+    y += step_y;
+    if (x >= snx) {
+      x -= snx;
+      y += 1;
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < kTransposeThin; ++k)
+    if (lane + k * G::kGroupThreads < n) *reinterpret_cast<T*>(tile + at[k]) = e[k];
+}
+
+template <class M, typename T>
+MMR_HD void transpose_store_element(const mmr_transpose_chunk& c, typename M::ptr dst, uint32_t b, const T* lds, uint32_t tid,
+                                    uint32_t x0, uint32_t y0, uint32_t snx, uint32_t sny) {
+  typedef TransposeTile<sizeof(T)> G;
+  const uint32_t wave = tid / G::kGroupThreads, lane = tid % G::kGroupThreads;
+  typename M::ptr d = dst + (b * c.dst_bstride + x0 * c.dst_xstride + static_cast<int64_t>(y0) * static_cast<int64_t>(sizeof(T)));
+  const uint8_t* tile = reinterpret_cast<const uint8_t*>(lds) + wave * G::kWaveLdsBytes;
+  const uint32_t n = snx * sny;
+  const uint32_t step_x = G::kGroupThreads / sny, step_y = G::kGroupThreads - step_x * sny;
+  uint32_t x = lane / sny, y = lane - x * sny;
+#pragma unroll
+  for (int k = 0; k < kTransposeThin; ++k) {
+    if (lane + k * G::kGroupThreads < n)
+      M::template storeu<T>(d + (x * c.dst_xstride + static_cast<int64_t>(y) * static_cast<int64_t>(sizeof(T))),
+                            *reinterpret_cast<const T*>(tile + transpose_lds_offset<sizeof(T)>(x, y)));
+    y += step_y;
+    x += step_x;
+    if (y >= sny) {
+      y -= sny;
+      x += 1;
+    }
+  }
+}
+
+// Thin path: a chunk whose tile is thinner than one vector one way (a small dimension moving into or out of the
+// minor position).  Its batch entries together fill at most the workgroup's LDS (the planner sizes nb so), so the
+// whole chunk moves in two phases around ONE workgroup barrier: every thread loads elements in source order
+// (batch entry, y, x: consecutive lanes read consecutive source elements) and parks them in LDS in destination
+// order (batch entry, x, y), then stores them in destination order (consecutive lanes write consecutive elements
+// of a destination row, and of the next row where the rows abut).  kTransposeThinUnroll loads of a lane are in
+// flight before its first LDS write; one division chain per phase, after that a lane's next element follows by a
+// fixed step with carries.
+constexpr int kTransposeThinUnroll = 8;
+
+MMR_HD bool transpose_is_thin(const mmr_transpose_chunk& c) {
+  const uint32_t vec = 16u / c.itemsize;
+  return c.nx < vec || c.ny < vec;
+}
+
+template <class M, typename T>
+MMR_HD void transpose_thin_load(const mmr_transpose_chunk& c, typename M::cptr src, T* lds, uint32_t tid) {
+  typedef TransposeTile<sizeof(T)> G;
+  const uint32_t nx = c.nx, ny = c.ny, tile = nx * ny, n = c.nb * tile;
+  const uint32_t step_x = G::kThreads % nx, rest = G::kThreads / nx, step_y = rest % ny, step_b = rest / ny;
+  uint32_t bb = tid / tile, y = (tid - bb * tile) / nx, x = tid - bb * tile - y * nx;
+  uint8_t* cells = reinterpret_cast<uint8_t*>(lds);
+  for (uint32_t base = tid; base < n; base += G::kThreads * kTransposeThinUnroll) {
+    T e[kTransposeThinUnroll];
+    uint32_t at[kTransposeThinUnroll];
+#pragma unroll
+    for (int k = 0; k < kTransposeThinUnroll; ++k) {
+      if (base + k * G::kThreads < n) {
+        e[k] = M::template loadu<T>(src + (bb * c.src_bstride + y * c.src_ystride +
+                                           static_cast<int64_t>(x) * static_cast<int64_t>(sizeof(T))));
+        at[k] = ((bb * nx + x) * ny + y) * static_cast<uint32_t>(sizeof(T));
+      }
+      x += step_x;
+      if (x >= nx) {
+        x -= nx;
+        y += 1;
+      }
+      y += step_y;
+      if (y >= ny) {
+        y -= ny;
+        bb += 1;
+      }
+      bb += step_b;
+    }
+#pragma unroll
+    for (int k = 0; k < kTransposeThinUnroll; ++k)
+      if (base + k * G::kThreads < n) *reinterpret_cast<T*>(cells + at[k]) = e[k];
   }
 }
 
 template <class M, typename T>
-MMR_HD void transpose_store(const mmr_transpose_chunk& c, typename M::ptr dst, uint32_t b, uint32_t sub, const T* lds, uint32_t tid) {
+MMR_HD void transpose_thin_store(const mmr_transpose_chunk& c, typename M::ptr dst, const T* lds, uint32_t tid) {
   typedef TransposeTile<sizeof(T)> G;
-  uint32_t x0, y0;
-  transpose_subtile<sizeof(T)>(sub, &x0, &y0);
-  if (x0 >= c.nx || y0 >= c.ny) return;
-  const uint32_t nx = c.nx - x0 < G::kEX ? c.nx - x0 : G::kEX, ny = c.ny - y0 < G::kEY ? c.ny - y0 : G::kEY;
-  typename M::ptr d = dst + (b * c.dst_bstride + x0 * c.dst_xstride + static_cast<int64_t>(y0) * static_cast<int64_t>(sizeof(T)));
-  const uint32_t n = nx * ny;
+  const uint32_t nx = c.nx, ny = c.ny, tile = nx * ny, n = c.nb * tile;
+  const uint32_t step_y = G::kThreads % ny, rest = G::kThreads / ny, step_x = rest % nx, step_b = rest / nx;
+  uint32_t bb = tid / tile, x = (tid - bb * tile) / ny, y = tid - bb * tile - x * ny;
   for (uint32_t i = tid; i < n; i += G::kThreads) {
-    const uint32_t x = i / ny, y = i - x * ny;
-    M::template storeu<T>(d + (x * c.dst_xstride + static_cast<int64_t>(y) * static_cast<int64_t>(sizeof(T))),
-                          lds[y * G::kPitch1 + x]);
+    M::template storeu<T>(dst + (bb * c.dst_bstride + x * c.dst_xstride + static_cast<int64_t>(y) * static_cast<int64_t>(sizeof(T))),
+                          lds[i]);
+    y += step_y;
+    if (y >= ny) {
+      y -= ny;
+      x += 1;
+    }
+    x += step_x;
+    if (x >= nx) {
+      x -= nx;
+      bb += 1;
+    }
+    bb += step_b;
+  }
+}
+
+// Phase 1 / phase 2 of batch entry b for thread tid, whatever its sub-tile needs.  `wave` = tid / kGroupThreads (the
+// kernel passes it as a wave-uniform value so the choice of path is a scalar branch).
+template <class M, typename T>
+MMR_HD void transpose_load_any(const mmr_transpose_chunk& c, typename M::cptr src, uint32_t b, T* lds, uint32_t tid,
+                               uint32_t wave) {
+  uint32_t x0, y0, snx, sny;
+  switch (transpose_mode<sizeof(T)>(c, wave, &x0, &y0, &snx, &sny)) {
+    case kTransposeVector: transpose_load_vec<M, T>(c, src, b, lds, tid); break;
+    case kTransposeGeneral: transpose_load_general<M, T>(c, src, b, lds, tid, x0, y0, snx, sny); break;
+    case kTransposeElement: transpose_load_element<M, T>(c, src, b, lds, tid, x0, y0, snx, sny); break;
+    default: break;
+  }
+}
+
+template <class M, typename T>
+MMR_HD void transpose_store_any(const mmr_transpose_chunk& c, typename M::ptr dst, uint32_t b, const T* lds, uint32_t tid,
+                                uint32_t wave) {
+  uint32_t x0, y0, snx, sny;
+  switch (transpose_mode<sizeof(T)>(c, wave, &x0, &y0, &snx, &sny)) {
+    case kTransposeVector: transpose_store_vec<M, T>(c, dst, b, lds, tid); break;
+    case kTransposeGeneral: transpose_store_general<M, T>(c, dst, b, lds, tid, x0, y0, snx, sny); break;
+    case kTransposeElement: transpose_store_element<M, T>(c, dst, b, lds, tid, x0, y0, snx, sny); break;
+    default: break;
   }
 }
 

@@ -37,9 +37,10 @@ struct DevicePlan {
   mmr_transpose_chunk* d_transposes = nullptr;
   struct TransposeRun {
     uint32_t itemsize;
+    bool vector_only;  // every chunk of the run satisfies transpose_is_vector
     int64_t begin, count;
   };
-  std::vector<TransposeRun> transpose_runs;  // the table is sorted by itemsize; one launch per run
+  std::vector<TransposeRun> transpose_runs;  // the table is sorted by (itemsize, kind); one launch per run
   bool tuned = false;                        // the table order has been chosen (timed or fixed by the options)
 
   DevicePlan() = default;
@@ -149,12 +150,21 @@ int make_device_plan(mmr_context* ctx, const std::vector<mmr_sharded_shape>& src
     uint32_t tile_x = 0, tile_y = 0;
     mmr::transpose_tile_extent(c.itemsize, &tile_x, &tile_y);
     const bool width_ok = c.itemsize == 1 || c.itemsize == 2 || c.itemsize == 4 || c.itemsize == 8 || c.itemsize == 16;
-    if (!width_ok || c.nx == 0 || c.ny == 0 || c.nx > tile_x || c.ny > tile_y)
+    if (!width_ok || c.nx == 0 || c.ny == 0)
+      return fail(MMR_INTERNAL, "transpose chunk %u x %u of %u-byte elements", c.nx, c.ny, c.itemsize);
+    if (mmr::transpose_is_thin(c)) {  // any shape, all batch entries in LDS at once
+      if (static_cast<uint64_t>(c.nb) * c.nx * c.ny * c.itemsize > mmr::kTransposeLdsBytes)
+        return fail(MMR_INTERNAL, "thin transpose chunk of %u x %u x %u elements exceeds the workgroup's LDS", c.nb, c.nx,
+                    c.ny);
+    } else if (c.nx > tile_x || c.ny > tile_y) {
       return fail(MMR_INTERNAL, "transpose chunk %u x %u of %u-byte elements does not fit the kernel's tile", c.nx, c.ny,
                   c.itemsize);
+    }
   }
   for (int64_t i = 0; i < static_cast<int64_t>(tr.size()); ++i) {
-    if (i == 0 || tr[i].itemsize != tr[i - 1].itemsize) dp->transpose_runs.push_back({tr[i].itemsize, i, 0});
+    const bool vec = mmr::transpose_is_vector(tr[i]);
+    if (i == 0 || tr[i].itemsize != tr[i - 1].itemsize || vec != dp->transpose_runs.back().vector_only)
+      dp->transpose_runs.push_back({tr[i].itemsize, vec, i, 0});
     dp->transpose_runs.back().count += 1;
   }
   if (int rc = upload(ctx, dp->plan.copy16, &dp->d_copy16)) return rc;
@@ -194,7 +204,7 @@ int launch_plan(mmr_context* ctx, const DevicePlan* dp, void* const* d_ptrs) {
   for (const DevicePlan::TransposeRun& run : dp->transpose_runs)
     // tiles are ordered in 8 x 8 blocks; runs of 64 table neighbours per XCD keep a block in one L2 (measured best)
     MMR_HIP(mmr::launch_transpose(dp->d_transposes + run.begin, run.count, d_ptrs, xm == 0 ? 64 : xm, run.itemsize,
-                                  ctx->stream));
+                                  run.vector_only, ctx->stream));
   return MMR_OK;
 }
 

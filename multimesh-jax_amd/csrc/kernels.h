@@ -22,9 +22,10 @@ hipError_t launch_copy16(const mmr_copy_chunk* d_chunks, int64_t n, void* const*
 hipError_t launch_copy_generic(const mmr_copy_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
                                hipStream_t stream);
 // LDS-staged tile transposes of elements of `itemsize` bytes (1, 2, 4, 8 or
-// 16); every chunk of the table must carry that itemsize.
+// 16); every chunk of the table must carry that itemsize, and with
+// `vector_only` every chunk must satisfy transpose_is_vector (chunk_ops.h).
 hipError_t launch_transpose(const mmr_transpose_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
-                            uint32_t itemsize, hipStream_t stream);
+                            uint32_t itemsize, bool vector_only, hipStream_t stream);
 
 }  // namespace mmr
 

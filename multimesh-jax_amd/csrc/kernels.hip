@@ -121,40 +121,88 @@ __device__ __forceinline__ void wave_sync() {
 }
 
 template <typename T>
+__device__ __forceinline__ void transpose_sync() {  // between the phases of the threads that share a sub-tile
+  if constexpr (TransposeTile<sizeof(T)>::kGroupThreads == 64) wave_sync(); else __syncthreads();
+}
+
+// VECTOR_ONLY: every chunk of the launch satisfies transpose_is_vector (the caller launches the two kinds apart).
+template <typename T, bool VECTOR_ONLY>
 __device__ __forceinline__ void transpose_tiles(const mmr_transpose_chunk& c, gcchar* src, gchar* dst, void* lds_raw) {
   typedef DeviceMem<true, true> M;
   typedef TransposeTile<sizeof(T)> G;
   T* lds = static_cast<T*>(lds_raw);
-  if (transpose_is_vector(c)) {  // uniform over the workgroup; waves run independently
+  const uint32_t tid = threadIdx.x;
+  // The threads that share a sub-tile take the same path, chosen by the part of the sub-tile that lies inside the
+  // tile; waves with sub-tiles of their own run independently (a sub-tile outside the tile: nothing to do).
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / G::kGroupThreads);
+  uint32_t x0, y0, snx, sny;
+  const TransposeMode mode = transpose_mode<sizeof(T)>(c, wave, &x0, &y0, &snx, &sny);
+  if constexpr (VECTOR_ONLY) {
+    if (mode == kTransposeNothing) return;
     for (uint32_t b = 0; b < c.nb; ++b) {
-      transpose_load_vec<M, T>(c, src, b, lds, threadIdx.x);
-      if constexpr (G::kGroupThreads == 64) wave_sync(); else __syncthreads();
-      transpose_store_vec<M, T>(c, dst, b, lds, threadIdx.x);
-      if constexpr (G::kGroupThreads == 64) wave_sync(); else __syncthreads();
+      transpose_load_vec<M, T>(c, src, b, lds, tid);
+      transpose_sync<T>();
+      transpose_store_vec<M, T>(c, dst, b, lds, tid);
+      transpose_sync<T>();
     }
     return;
   }
-  for (uint32_t b = 0; b < c.nb; ++b) {
-    for (uint32_t sub = 0; sub < G::kWaves; ++sub) {
-      transpose_load<M, T>(c, src, b, sub, lds, threadIdx.x);
-      __syncthreads();
-      transpose_store<M, T>(c, dst, b, sub, lds, threadIdx.x);
-      __syncthreads();
-    }
+  if (transpose_is_thin(c)) {  // uniform over the workgroup: the whole chunk in two phases around one barrier
+    transpose_thin_load<M, T>(c, src, lds, tid);
+    __syncthreads();
+    transpose_thin_store<M, T>(c, dst, lds, tid);
+    return;
+  }
+  // One batch loop per path: with the choice inside a common loop the compiler hoists every path's loop-invariant
+  // addresses out of it and the register need is the sum over the paths instead of the maximum.
+  switch (mode) {
+    case kTransposeVector:
+      for (uint32_t b = 0; b < c.nb; ++b) {
+        transpose_load_vec<M, T>(c, src, b, lds, tid);
+        transpose_sync<T>();
+        transpose_store_vec<M, T>(c, dst, b, lds, tid);
+        transpose_sync<T>();
+      }
+      break;
+    case kTransposeGeneral:
+      for (uint32_t b = 0; b < c.nb; ++b) {
+        transpose_load_general<M, T>(c, src, b, lds, tid, x0, y0, snx, sny);
+        transpose_sync<T>();
+        transpose_store_general<M, T>(c, dst, b, lds, tid, x0, y0, snx, sny);
+        transpose_sync<T>();
+      }
+      break;
+    case kTransposeElement:
+      for (uint32_t b = 0; b < c.nb; ++b) {
+        transpose_load_element<M, T>(c, src, b, lds, tid, x0, y0, snx, sny);
+        transpose_sync<T>();
+        transpose_store_element<M, T>(c, dst, b, lds, tid, x0, y0, snx, sny);
+        transpose_sync<T>();
+      }
+      break;
+    default:  // the sub-tile lies outside the tile (never the case where the whole workgroup shares one sub-tile)
+      break;
   }
 }
 
+// Waves per SIMD the register allocation of the general kernel aims at (0 = the compiler's choice): three where the
+// widest path fits 168 registers without spilling; the 2-byte instance needs 170 and stays at two.
 template <typename T>
-__global__ __launch_bounds__(TransposeTile<sizeof(T)>::kThreads) void mmr_transpose_kernel(
+constexpr int transpose_general_waves() { return sizeof(T) == 2 || sizeof(T) >= 8 ? 0 : 3; }
+
+template <typename T, bool VECTOR_ONLY>
+__global__ __launch_bounds__(TransposeTile<sizeof(T)>::kThreads, VECTOR_ONLY ? 0 : transpose_general_waves<T>())
+void mmr_transpose_kernel(
     const mmr_transpose_chunk* __restrict__ chunks, uint32_t n, void* const* __restrict__ ptrs, uint32_t xcd_group) {
-  // one instance per element width, each with the register and LDS budget of its own tile (32 KiB of LDS)
-  __shared__ __attribute__((aligned(16))) uint8_t lds[TransposeTile<sizeof(T)>::kLdsBytes];
+  // one instance per element width, each with the register and LDS budget of its own tile; the general kernel
+  // also takes thin chunks, which park up to kTransposeLdsBytes at once
+  __shared__ __attribute__((aligned(16))) uint8_t lds[VECTOR_ONLY ? TransposeTile<sizeof(T)>::kLdsBytes : kTransposeLdsBytes];
   const uint32_t ci = chunk_index(blockIdx.x, xcd_group);
   if (ci >= n) return;  // uniform over the workgroup: no barrier is skipped by part of it
   const mmr_transpose_chunk c = chunks[ci];
   gcchar* src = slot_base(ptrs, c.src_slot, c.src_off);
   gchar* dst = slot_base(ptrs, c.dst_slot, c.dst_off);
-  transpose_tiles<T>(c, src, dst, lds);
+  transpose_tiles<T, VECTOR_ONLY>(c, src, dst, lds);
 }
 
 // Flat copy of `vectors` 16-byte vectors: workgroup i moves the i-th block of kFlatVectors vectors, all loads of a
@@ -225,23 +273,26 @@ hipError_t launch_copy_generic(const mmr_copy_chunk* d_chunks, int64_t n, void* 
 
 template <typename T>
 hipError_t launch_transpose_of(const mmr_transpose_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
-                               hipStream_t stream) {
+                               bool vector_only, hipStream_t stream) {
   const uint32_t group = xcd_group_of(n, xcd_mode);
-  hipLaunchKernelGGL(mmr_transpose_kernel<T>, dim3(grid_size(n, group)), dim3(TransposeTile<sizeof(T)>::kThreads), 0, stream,
-                     d_chunks, static_cast<uint32_t>(n), d_ptrs, group);
+  const dim3 grid(grid_size(n, group)), block(TransposeTile<sizeof(T)>::kThreads);
+  if (vector_only)
+    hipLaunchKernelGGL((mmr_transpose_kernel<T, true>), grid, block, 0, stream, d_chunks, static_cast<uint32_t>(n), d_ptrs, group);
+  else
+    hipLaunchKernelGGL((mmr_transpose_kernel<T, false>), grid, block, 0, stream, d_chunks, static_cast<uint32_t>(n), d_ptrs, group);
   return hipGetLastError();
 }
 
 hipError_t launch_transpose(const mmr_transpose_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
-                            uint32_t itemsize, hipStream_t stream) {
+                            uint32_t itemsize, bool vector_only, hipStream_t stream) {
   if (n == 0) return hipSuccess;
   if (hipError_t e = check_grid(n)) return e;
   switch (itemsize) {
-    case 1: return launch_transpose_of<uint8_t>(d_chunks, n, d_ptrs, xcd_mode, stream);
-    case 2: return launch_transpose_of<uint16_t>(d_chunks, n, d_ptrs, xcd_mode, stream);
-    case 4: return launch_transpose_of<uint32_t>(d_chunks, n, d_ptrs, xcd_mode, stream);
-    case 8: return launch_transpose_of<uint64_t>(d_chunks, n, d_ptrs, xcd_mode, stream);
-    case 16: return launch_transpose_of<V16>(d_chunks, n, d_ptrs, xcd_mode, stream);
+    case 1: return launch_transpose_of<uint8_t>(d_chunks, n, d_ptrs, xcd_mode, vector_only, stream);
+    case 2: return launch_transpose_of<uint16_t>(d_chunks, n, d_ptrs, xcd_mode, vector_only, stream);
+    case 4: return launch_transpose_of<uint32_t>(d_chunks, n, d_ptrs, xcd_mode, vector_only, stream);
+    case 8: return launch_transpose_of<uint64_t>(d_chunks, n, d_ptrs, xcd_mode, vector_only, stream);
+    case 16: return launch_transpose_of<V16>(d_chunks, n, d_ptrs, xcd_mode, vector_only, stream);
     default: return hipErrorInvalidValue;
   }
 }

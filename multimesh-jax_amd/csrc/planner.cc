@@ -222,8 +222,24 @@ class Builder {
                        int x, int y, int itemsize) {
     uint32_t tx = 0, ty = 0;
     transpose_tile_extent(static_cast<uint32_t>(itemsize), &tx, &ty);
-    const int64_t tile_x = tx, tile_y = ty;
+    int64_t tile_x = tx, tile_y = ty;
     const BoxDim dx = dims[x], dy = dims[y];
+    // A box thinner than one 16-byte vector one way (3 channels moving out of the minor position, say) goes through
+    // the kernel's thin path, which takes any tile that fits the workgroup's LDS: make the tile long the other way
+    // instead of leaving chunks of a few hundred bytes.  That path works element by element, so its chunks are
+    // sized by elements (32 per thread at most), and a small box is cut into about a thousand chunks or more so
+    // that it still spreads over the 256 CUs.
+    const int64_t vec = 16 / itemsize;
+    const bool thin = dx.n < vec || dy.n < vec;
+    int64_t chunk_bytes = kTransposeChunkBytes;
+    if (thin) {
+      int64_t box_bytes = itemsize;
+      for (const BoxDim& d : dims) box_bytes *= d.n;
+      chunk_bytes = std::min<int64_t>(chunk_bytes, 8192 * itemsize);
+      chunk_bytes = std::max<int64_t>(std::min<int64_t>(chunk_bytes, box_bytes / 1024), 1024);
+      if (dx.n < vec) tile_y = std::max<int64_t>(tile_y, chunk_bytes / (dx.n * itemsize) / tile_y * tile_y);
+      else tile_x = std::max<int64_t>(tile_x, chunk_bytes / (dy.n * itemsize) / tile_x * tile_x);
+    }
     std::vector<BoxDim> outer;
     for (int i = 0; i < static_cast<int>(dims.size()); ++i)
       if (i != x && i != y) outer.push_back(dims[i]);
@@ -235,7 +251,7 @@ class Builder {
     }
     // tiles narrower than the workgroup tile (a short x or y extent) are batched along the next dimension
     const int64_t tile_bytes = std::min(tile_x, dx.n) * std::min(tile_y, dy.n) * itemsize;
-    const int64_t nb = std::max<int64_t>(1, std::min<int64_t>(db.n, kTransposeChunkBytes / tile_bytes));
+    const int64_t nb = std::max<int64_t>(1, std::min<int64_t>(db.n, chunk_bytes / tile_bytes));
     for_each_index(outer, [&](int64_t ds, int64_t dd) {
       for (int64_t b0 = 0; b0 < db.n; b0 += nb) {
         for (int64_t y0 = 0; y0 < dy.n; y0 += tile_y) {
@@ -480,10 +496,13 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
                                          : std::make_pair(a.src_slot, a.src_off) < std::make_pair(b.src_slot, b.src_off);
                      });
   }
-  // one launch per element width (a narrow type's kernel keeps its own register and LDS budget): runs of equal
-  // itemsize, the order above kept inside each run
+  // one launch per element width (a narrow type's kernel keeps its own register and LDS budget) and kind (tiles that
+  // are 16-byte aligned with whole vectors on both sides run through a leaner kernel than ragged or misaligned
+  // ones): runs of equal (itemsize, kind), the order above kept inside each run
   std::stable_sort(plan->transposes.begin(), plan->transposes.end(),
-                   [](const mmr_transpose_chunk& a, const mmr_transpose_chunk& b) { return a.itemsize < b.itemsize; });
+                   [](const mmr_transpose_chunk& a, const mmr_transpose_chunk& b) {
+                     return std::make_pair(a.itemsize, !transpose_is_vector(a)) < std::make_pair(b.itemsize, !transpose_is_vector(b));
+                   });
   plan->stats.order_used = options.order;
   plan->stats.interleave_kib = options.order == 4 ? (((options.flags >> 8) & 0xffffu) ? ((options.flags >> 8) & 0xffffu) : 64) : 0;
   plan->stats.n_arrays = n;

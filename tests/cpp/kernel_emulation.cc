@@ -83,18 +83,24 @@ void run_transpose(const mmr_transpose_chunk& c, const uint8_t* src, uint8_t* ds
   alignas(16) static thread_local uint8_t lds_raw[mmr::kTransposeLdsBytes];
   static_assert(G::kLdsBytes <= mmr::kTransposeLdsBytes, "LDS tile too large");
   T* lds = reinterpret_cast<T*>(lds_raw);
-  // a phase runs for every thread before the next one starts: what the wave fence (vector path) or the
-  // workgroup barrier (element path) guarantees on the device
+  // a phase runs for every thread before the next one starts: what the wave fence (or the workgroup barrier
+  // where the waves share a sub-tile) guarantees on the device
+  if (!mmr::transpose_is_vector(c) && mmr::transpose_is_thin(c)) {  // as the general kernel decides
+    std::memset(lds_raw, 0xA5, sizeof(lds_raw));
+    if (static_cast<uint64_t>(c.nb) * c.nx * c.ny * sizeof(T) > sizeof(lds_raw)) {
+      g_error = "thin transpose chunk larger than the workgroup's LDS";
+      return;
+    }
+    for (uint32_t tid = 0; tid < kThreads; ++tid) mmr::transpose_thin_load<HostMem, T>(c, src, lds, tid);
+    for (uint32_t tid = 0; tid < kThreads; ++tid) mmr::transpose_thin_store<HostMem, T>(c, dst, lds, tid);
+    return;
+  }
   for (uint32_t b = 0; b < c.nb; ++b) {
-    if (mmr::transpose_is_vector(c)) {
-      for (uint32_t tid = 0; tid < kThreads; ++tid) mmr::transpose_load_vec<HostMem, T>(c, src, b, lds, tid);
-      for (uint32_t tid = 0; tid < kThreads; ++tid) mmr::transpose_store_vec<HostMem, T>(c, dst, b, lds, tid);
-      continue;
-    }
-    for (uint32_t sub = 0; sub < G::kWaves; ++sub) {
-      for (uint32_t tid = 0; tid < kThreads; ++tid) mmr::transpose_load<HostMem, T>(c, src, b, sub, lds, tid);
-      for (uint32_t tid = 0; tid < kThreads; ++tid) mmr::transpose_store<HostMem, T>(c, dst, b, sub, lds, tid);
-    }
+    std::memset(lds_raw, 0xA5 ^ static_cast<int>(b & 0x3f), sizeof(lds_raw));  // a cell read before it is written shows up as wrong bytes
+    for (uint32_t tid = 0; tid < kThreads; ++tid)
+      mmr::transpose_load_any<HostMem, T>(c, src, b, lds, tid, tid / G::kGroupThreads);
+    for (uint32_t tid = 0; tid < kThreads; ++tid)
+      mmr::transpose_store_any<HostMem, T>(c, dst, b, lds, tid, tid / G::kGroupThreads);
   }
 }
 
@@ -196,7 +202,7 @@ int mmr_emulate_plan(const mmr_plan* plan, void* const* slot_ptrs, const size_t*
       uint8_t* dst = base(c.dst_slot, c.dst_off);
       uint32_t tile_x = 0, tile_y = 0;
       mmr::transpose_tile_extent(c.itemsize, &tile_x, &tile_y);
-      if (c.nx > tile_x || c.ny > tile_y) {
+      if (!mmr::transpose_is_thin(c) && (c.nx > tile_x || c.ny > tile_y)) {  // thin chunks: checked against LDS below
         g_error = "transpose tile larger than the LDS tile";
         return;
       }

@@ -192,6 +192,44 @@ def test_transpose_kernel_large(ctx, type_):
     _compare([a], [g], gpu_reshard(ctx, [a], [g]))
 
 
+@pytest.mark.parametrize("type_", ["U8", "BF16", "F32", "F64", "C128"])
+def test_transpose_ragged_and_misaligned_tiles(ctx, type_):
+    """Transposed layouts whose tiles are not 16-byte aligned or do not hold whole vectors (unaligned accesses,
+    vectors slid inwards at the edges, sub-tiles thinner than a vector), and one large odd-sized array."""
+    item = ro.ITEMSIZE[type_]
+    rng = np.random.Generator(np.random.PCG64(41))
+    for shape, st_, dt_ in (((250, 381), (2, 1), (1, 3)), ((135, 203), (1, 1), (1, 1)), ((129, 257), (1, 2), (2, 1)),
+                            ((20, 300), (1, 1), (1, 1)), ((300, 20), (1, 1), (1, 1)), ((3, 500), (1, 1), (1, 1)),
+                            ((2046, 1027), (2, 1), (1, 2))):
+        say("ragged transpose %s %r" % (type_, shape))
+        ns = st_[0] * st_[1]
+        a = {"name": "t", "type": type_, "shape": shape,
+             "src": {"dims": [(shape[0], st_[0], 0), (shape[1], st_[1], 1)], "dev_start": 0, "dev_count": ns},
+             "dst": {"dims": [(shape[0], dt_[0], 0), (shape[1], dt_[1], 1)], "dev_start": ns,
+                     "dev_count": dt_[0] * dt_[1], "minor_to_major": [0, 1]},
+             "seed": 0, "dist": "raw"}
+        g = rng.integers(0, 256, size=int(np.prod(shape)) * item, dtype=np.uint8).view(ro.raw_dtype(type_)).reshape(shape)
+        _compare([a], [g], gpu_reshard(ctx, [a], [g]))
+
+
+@pytest.mark.parametrize("type_", ["U8", "BF16", "F32", "F64"])
+def test_transpose_thin_tiles(ctx, type_):
+    """A dimension of a few elements moving into or out of the minor position (3 channels, 6 heads): boxes thinner
+    than one 16-byte vector take the kernel's thin path, with tiles as long as the workgroup's LDS allows."""
+    item = ro.ITEMSIZE[type_]
+    rng = np.random.Generator(np.random.PCG64(47))
+    for shape, m2m in (((40, 700, 3), [1, 0, 2]), ((50, 6, 1030), [1, 2, 0]), ((7, 1, 33000), [1, 0, 2]),
+                       ((300, 2000, 3), [1, 0, 2])):
+        say("thin transpose %s %r" % (type_, shape))
+        a = {"name": "t", "type": type_, "shape": shape,
+             "src": {"dims": [(n, 1, i) for i, n in enumerate(shape)], "dev_start": 0, "dev_count": 1},
+             "dst": {"dims": [(n, 1, i) for i, n in enumerate(shape)], "dev_start": 1, "dev_count": 1,
+                     "minor_to_major": m2m},
+             "seed": 0, "dist": "raw"}
+        g = rng.integers(0, 256, size=int(np.prod(shape)) * item, dtype=np.uint8).view(ro.raw_dtype(type_)).reshape(shape)
+        _compare([a], [g], gpu_reshard(ctx, [a], [g]))
+
+
 def test_python_test_toy_shapes(ctx):
     """The shapes the reference's end-to-end Python tests reshard: (4,4) and (8,4)
     f32 between two 2-device meshes and from 4 devices onto 2+2."""

@@ -97,7 +97,7 @@ def test_ragged_rows_through_the_kernel_code(a, chunk_bytes, shape):
 @pytest.mark.parametrize("type_", ["U8", "BF16", "F32", "F64", "C128"])
 @pytest.mark.parametrize("shape", [(256, 384), (192, 200), (130, 256)])
 def test_transposed_layout_vector_and_element_tiles(type_, shape):
-    """Aligned tiles take the 16-byte vector path, ragged edge tiles the element path."""
+    """Aligned tiles take the 16-byte vector path, ragged edge tiles the general path."""
     from oracle import reshard_oracle as ro
     item = ro.ITEMSIZE[type_]
     a = {"name": "t", "type": type_, "shape": shape,
@@ -108,6 +108,63 @@ def test_transposed_layout_vector_and_element_tiles(type_, shape):
     g = rng.integers(0, 256, size=int(np.prod(shape)) * item, dtype=np.uint8).view(ro.raw_dtype(type_)).reshape(shape)
     plan = _check([a], [g])
     assert plan.stats["n_transpose_chunks"] > 0
+
+
+@pytest.mark.parametrize("type_", ["U8", "BF16", "F32", "F64", "C128"])
+@pytest.mark.parametrize("shape,src_tiles,dst_tiles", [
+    ((250, 381), (2, 1), (1, 3)),   # odd row lengths: no stride is a multiple of 16 -> general path everywhere;
+                                    # vectors cut off by the tile edge slide inwards on both sides
+    ((135, 203), (1, 1), (1, 1)),   # one full sub-tile, one ragged, one thinner than a vector (element path)
+    ((67, 131), (1, 1), (1, 1)),    # 3 columns past the first sub-tile
+    ((129, 257), (1, 2), (2, 1)),   # a single row / column beyond full tiles
+    ((20, 300), (1, 1), (1, 1)),    # short in y (packed source rows run past the edge)
+    ((300, 20), (1, 1), (1, 1)),    # short in x
+    ((3, 500), (1, 1), (1, 1)),     # thinner than one vector of any type but C128
+])
+def test_transposed_layout_ragged_and_misaligned_tiles(type_, shape, src_tiles, dst_tiles):
+    """Tiles that are not 16-byte aligned or do not hold whole vectors: unaligned 16-byte accesses with vectors
+    slid inwards at the edges, element by element only where a sub-tile is thinner than one vector."""
+    from oracle import reshard_oracle as ro
+    item = ro.ITEMSIZE[type_]
+    ns = src_tiles[0] * src_tiles[1]
+    a = {"name": "t", "type": type_, "shape": shape,
+         "src": {"dims": [(shape[0], src_tiles[0], 0), (shape[1], src_tiles[1], 1)], "dev_start": 0, "dev_count": ns},
+         "dst": {"dims": [(shape[0], dst_tiles[0], 0), (shape[1], dst_tiles[1], 1)], "dev_start": ns,
+                 "dev_count": dst_tiles[0] * dst_tiles[1], "minor_to_major": [0, 1]},
+         "seed": 0, "dist": "raw"}
+    rng = np.random.Generator(np.random.PCG64(37))
+    g = rng.integers(0, 256, size=int(np.prod(shape)) * item, dtype=np.uint8).view(ro.raw_dtype(type_)).reshape(shape)
+    plan = _check([a], [g])
+    assert plan.stats["n_transpose_chunks"] > 0
+
+
+@pytest.mark.parametrize("type_", ["U8", "BF16", "F32", "F64"])
+@pytest.mark.parametrize("shape,m2m", [
+    ((40, 700, 3), [1, 0, 2]),    # 3 channels leave the minor position: x extent 3, tiles thousands of elements long in y
+    ((50, 6, 1030), [1, 2, 0]),   # a dim of 6 becomes the minor one: y extent 6
+    ((7, 1, 33000), [1, 0, 2]),
+])
+def test_transposed_layout_thin_tiles(type_, shape, m2m):
+    """A box thinner than one 16-byte vector one way: the whole chunk (tiles as long as the workgroup's LDS
+    allows) moves in two phases around one workgroup barrier."""
+    from oracle import reshard_oracle as ro
+    import multimesh_jax_amd as mm
+    from helpers import lib_shape
+    item = ro.ITEMSIZE[type_]
+    a = {"name": "t", "type": type_, "shape": shape,
+         "src": {"dims": [(n, 1, i) for i, n in enumerate(shape)], "dev_start": 0, "dev_count": 1},
+         "dst": {"dims": [(n, 1, i) for i, n in enumerate(shape)], "dev_start": 1, "dev_count": 1, "minor_to_major": m2m},
+         "seed": 0, "dist": "raw"}
+    rng = np.random.Generator(np.random.PCG64(43))
+    g = rng.integers(0, 256, size=int(np.prod(shape)) * item, dtype=np.uint8).view(ro.raw_dtype(type_)).reshape(shape)
+    plan = _check([a], [g])
+    t = plan.transpose_chunks()
+    if shape[1] != 1:
+        assert len(t) > 0
+        vec = 16 // item
+        thin = (t["nx"] < vec) | (t["ny"] < vec)
+        if thin.any():  # (F64 has 2-element vectors: 3 channels are not thin there)
+            assert (t["nb"].astype(np.int64) * t["nx"] * t["ny"] * item)[thin].max() <= 32 * 1024
 
 
 def test_transposed_benchmark_workloads_scaled():
