@@ -72,7 +72,13 @@ def measure(ctx, mm, workloads, args, config, with_parity=True):
         arrays = [a for a in arrays if args.name in a["name"]]
     gs = [workloads.generate(a) for a in arrays]
     alg_bytes = workloads.algorithmic_bytes(arrays)
-    sets = [make_stores(ctx, arrays, gs, poison=None) for _ in range(max(1, args.sets))]
+    # Buffer sets rotated between steps: at least `--sets`, and enough of them that 768 MiB of other buffers are
+    # touched before a set comes round again - the 256 MB Infinity Cache must not serve a small configuration's reads
+    # (an explicit --sets 1 or 2 is a probing run and is taken as given).
+    n_sets = max(1, args.sets)
+    if args.sets >= 3:
+        n_sets = max(n_sets, -(-(768 << 20) // max(alg_bytes, 1)) + 1)
+    sets = [make_stores(ctx, arrays, gs, poison=None) for _ in range(n_sets)]
 
     def step(i):
         srcs, dsts = sets[i % len(sets)]

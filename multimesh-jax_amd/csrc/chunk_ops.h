@@ -61,68 +61,55 @@ inline uint32_t grid_size(int64_t n, uint32_t group) {
 
 // ---------------------------------------------------------------------------
 // Aligned copy: every offset, stride and row width is a multiple of 16 bytes.
-// Rows of wv = w/16 vectors.  No division in the loops: a thread fixes its
-// column (and, for rows narrower than the workgroup, its sub-row) once, then
-// steps through rows.  UNROLL loads are issued before the first store.
+// Rows of wv = w/16 vectors.  The (row, column) pairs of the chunk are numbered
+// row after row and dealt to the lanes, UNROLL per lane and pass.  Branch-free:
+// a lane whose number runs past the end of the chunk repeats the chunk's last
+// vector (same load, same store as the rightful lane), so a pass is
+// straight-line code - UNROLL loads, UNROLL stores, the next pass's loads
+// issued while these stores are still in flight - where per-lane branches made
+// the compiler wait for each access before issuing the next.  One division
+// chain per thread; after that a lane's (r2, r1, column) advances by a fixed
+// step with carries.
 // ---------------------------------------------------------------------------
-template <class M, int THREADS, int UNROLL>
-MMR_HD void copy16_chunk(const mmr_copy_chunk& c, typename M::cptr src, typename M::ptr dst, uint32_t tid) {
-  const bool fill = c.src_slot == MMR_SLOT_FILL;
-  const uint32_t wv = c.w >> 4;
-  const uint32_t rows = c.n1 * c.n2;
-  if (wv >= THREADS) {
-    // wide rows: the whole workgroup walks one row at a time
-    for (uint32_t r2 = 0; r2 < c.n2; ++r2) {
-      for (uint32_t r1 = 0; r1 < c.n1; ++r1) {
-        typename M::cptr srow = src + (r2 * c.s2 + r1 * c.s1);
-        typename M::ptr drow = dst + (r2 * c.d2 + r1 * c.d1);
-        for (uint32_t c0 = tid; c0 < wv; c0 += THREADS * UNROLL) {
-          V16 v[UNROLL];
-#pragma unroll
-          for (int u = 0; u < UNROLL; ++u) {
-            const uint32_t col = c0 + u * THREADS;
-            if (col < wv) v[u] = fill ? V16{0, 0, 0, 0} : M::load16(srow + (static_cast<int64_t>(col) << 4));
-          }
-#pragma unroll
-          for (int u = 0; u < UNROLL; ++u) {
-            const uint32_t col = c0 + u * THREADS;
-            if (col < wv) M::store16(drow + (static_cast<int64_t>(col) << 4), v[u]);
-          }
-        }
-      }
-    }
-    return;
-  }
-  // narrow rows: R = THREADS / wv rows per pass; thread = (sub-row, column), fixed
-  const uint32_t R = THREADS / wv;
-  const uint32_t sub = tid / wv;
-  const uint32_t col = tid - sub * wv;
-  if (sub >= R) return;
-  const int64_t cb = static_cast<int64_t>(col) << 4;
-  // (r2, r1) of this thread's first row and the per-pass step, so the loop needs no division
-  uint32_t r2 = sub / c.n1, r1 = sub - r2 * c.n1;
-  const uint32_t step2 = R / c.n1, step1 = R - step2 * c.n1;
-  for (uint32_t row0 = sub; row0 < rows; row0 += R * UNROLL) {
+template <class M, int THREADS, int UNROLL, bool FILL>
+MMR_HD void copy16_rows(const mmr_copy_chunk& c, typename M::cptr src, typename M::ptr dst, uint32_t tid) {
+  const uint32_t wv = c.w >> 4, n1 = c.n1, n2 = c.n2;
+  const uint32_t total = n1 * n2 * wv;
+  const uint32_t step_col = THREADS % wv, rest = THREADS / wv, step_r1 = rest % n1, step_r2 = rest / n1;
+  uint32_t row = tid / wv, col = tid - row * wv, r2 = row / n1, r1 = row - r2 * n1;
+  for (uint32_t base = 0; base < total; base += THREADS * UNROLL) {
     V16 v[UNROLL];
-    int64_t doff[UNROLL];
+    int64_t soff[UNROLL], doff[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      if (row0 + u * R < rows) {
-        doff[u] = r2 * c.d2 + r1 * c.d1 + cb;
-        v[u] = fill ? V16{0, 0, 0, 0} : M::load16(src + (r2 * c.s2 + r1 * c.s1 + cb));
+      const bool inside = base + tid + u * THREADS < total;
+      const uint32_t q2 = inside ? r2 : n2 - 1, q1 = inside ? r1 : n1 - 1, qc = inside ? col : wv - 1;
+      soff[u] = q2 * c.s2 + q1 * c.s1 + (static_cast<int64_t>(qc) << 4);
+      doff[u] = q2 * c.d2 + q1 * c.d1 + (static_cast<int64_t>(qc) << 4);
+      col += step_col;
+      if (col >= wv) {
+        col -= wv;
+        r1 += 1;
       }
-      r1 += step1;
-      r2 += step2;
-      if (r1 >= c.n1) {
-        r1 -= c.n1;
+      r1 += step_r1;
+      if (r1 >= n1) {
+        r1 -= n1;
         r2 += 1;
       }
+      r2 += step_r2;
     }
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      if (row0 + u * R < rows) M::store16(dst + doff[u], v[u]);
-    }
+    for (int u = 0; u < UNROLL; ++u) v[u] = FILL ? V16{0, 0, 0, 0} : M::load16(src + soff[u]);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) M::store16(dst + doff[u], v[u]);
   }
+}
+
+template <class M, int THREADS, int UNROLL>
+MMR_HD void copy16_chunk(const mmr_copy_chunk& c, typename M::cptr src, typename M::ptr dst, uint32_t tid) {
+  // uniform over the workgroup; a chunk without a source writes zeros
+  if (c.src_slot == MMR_SLOT_FILL) copy16_rows<M, THREADS, UNROLL, true>(c, src, dst, tid);
+  else copy16_rows<M, THREADS, UNROLL, false>(c, src, dst, tid);
 }
 
 // ---------------------------------------------------------------------------
@@ -137,7 +124,8 @@ MMR_HD void copy16_chunk(const mmr_copy_chunk& c, typename M::cptr src, typename
 // slides inwards until it lies inside the row: it still moves 16 bytes, now
 // unaligned on both sides, and overlaps its neighbour, which writes the same
 // values to the shared bytes.  So every lane runs the same two instructions
-// and no access ever leaves its row.  Rows
+// and no access ever leaves its row (lanes with no pair of their own left
+// repeat the last pair, see generic_slot).  Rows
 // narrower than 16 bytes have no room to slide: their 1..15 bytes move as
 // 8/4/2/1-byte pieces (binary decomposition of the length), carried in one V16:
 // .x/.y the 8-byte piece, .z the 4-byte piece, .w the 2-byte piece (low half)
@@ -167,61 +155,43 @@ MMR_HD void store_ragged(typename M::ptr d, uint32_t len, V16 v) {
   if (len & 1) M::template storeu<uint8_t>(d + o1, static_cast<uint8_t>(v.w >> 16));
 }
 
-// One (row, slot) of a generic chunk: phase 1 (all loads).  WIDE: rows of at least 16 bytes.
-template <class M, bool WIDE>
-MMR_HD void generic_load(const mmr_copy_chunk& c, typename M::cptr src, typename M::ptr dst, bool fill, uint32_t row,
-                         uint32_t slot, V16* v, typename M::ptr* dpos, int32_t* len) {
+// Rows of at least 16 bytes.  Branch-free: a (row, slot) pair past the end of its row or of the chunk repeats the
+// last slot of that row (of the last row), i.e. loads the same 16 bytes and stores them to the same place as the
+// rightful lane does.  With no lane predicated the loop body is straight-line code - UNROLL loads, one wait,
+// UNROLL stores - where per-lane branches made the compiler wait for each access before issuing the next.
+template <class M>
+MMR_HD void generic_slot(const mmr_copy_chunk& c, typename M::cptr src, typename M::ptr dst, bool fill, uint32_t row,
+                         uint32_t slot, typename M::cptr* spos, typename M::ptr* dpos) {
   typename M::ptr drow = dst + row * c.d1;
   typename M::cptr srow = src + row * c.s1;
   const int32_t w = static_cast<int32_t>(c.w);
   const int32_t mis = static_cast<int32_t>((fill ? M::addr(drow) : M::caddr(srow)) & 15u);
   const int32_t rel = static_cast<int32_t>(slot << 4) - mis;  // row-relative byte where this aligned slot starts
-  if constexpr (WIDE) {
-    if (rel >= w) {
-      *len = 0;
-      return;
-    }
-    const int32_t lo = rel < 0 ? 0 : (rel + 16 > w ? w - 16 : rel);
-    *len = 16;
-    *dpos = drow + lo;
-    *v = fill ? V16{0, 0, 0, 0} : M::load16u(srow + lo);
-  } else {
-    const int32_t lo = rel < 0 ? 0 : rel;
-    const int32_t hi = rel + 16 < w ? rel + 16 : w;
-    *len = hi - lo;
-    *dpos = drow + lo;
-    if (*len > 0) *v = fill ? V16{0, 0, 0, 0} : load_ragged<M>(srow + lo, static_cast<uint32_t>(*len));
-  }
+  const int32_t lo = rel < 0 ? 0 : (rel + 16 > w ? w - 16 : rel);
+  *spos = srow + lo;
+  *dpos = drow + lo;
 }
 
-template <class M, bool WIDE>
-MMR_HD void generic_store(typename M::ptr dpos, int32_t len, V16 v) {
-  if constexpr (WIDE) {
-    if (len != 0) M::template storeu<V16>(dpos, v);
-  } else {
-    if (len > 0) store_ragged<M>(dpos, static_cast<uint32_t>(len), v);
-  }
-}
-
-template <class M, int THREADS, int UNROLL, bool WIDE>
-MMR_HD void generic_rows(const mmr_copy_chunk& c, typename M::cptr src, typename M::ptr dst, uint32_t tid) {
-  const bool fill = c.src_slot == MMR_SLOT_FILL;
+template <class M, int THREADS, int UNROLL, bool FILL>
+MMR_HD void generic_wide_rows(const mmr_copy_chunk& c, typename M::cptr src, typename M::ptr dst, uint32_t tid) {
+  constexpr bool fill = FILL;  // a chunk without a source writes zeros: its own instance, so neither loop branches
   const uint32_t slots = ((c.w + 15u) >> 4) + 1u;  // a row of w bytes touches at most this many aligned slots
   const uint32_t rows = c.n1;
   if (slots >= THREADS) {
     for (uint32_t row = 0; row < rows; ++row) {
-      for (uint32_t s0 = tid; s0 < slots; s0 += THREADS * UNROLL) {
+      for (uint32_t s0 = 0; s0 < slots; s0 += THREADS * UNROLL) {
         V16 v[UNROLL];
+        typename M::cptr spos[UNROLL];
         typename M::ptr dpos[UNROLL];
-        int32_t len[UNROLL];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
-          len[u] = 0;
-          const uint32_t slot = s0 + u * THREADS;
-          if (slot < slots) generic_load<M, WIDE>(c, src, dst, fill, row, slot, &v[u], &dpos[u], &len[u]);
+          const uint32_t slot = s0 + tid + u * THREADS;
+          generic_slot<M>(c, src, dst, fill, row, slot < slots ? slot : slots - 1, &spos[u], &dpos[u]);
         }
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) generic_store<M, WIDE>(dpos[u], len[u], v[u]);
+        for (int u = 0; u < UNROLL; ++u) v[u] = fill ? V16{0, 0, 0, 0} : M::load16u(spos[u]);
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) M::template storeu<V16>(dpos[u], v[u]);
       }
     }
     return;
@@ -232,14 +202,14 @@ MMR_HD void generic_rows(const mmr_copy_chunk& c, typename M::cptr src, typename
   const uint32_t total = rows * slots;
   const uint32_t step_rows = THREADS / slots, step_slots = THREADS - step_rows * slots;
   uint32_t row = tid / slots, slot = tid - row * slots;
-  for (uint32_t i0 = tid; i0 < total; i0 += THREADS * UNROLL) {
+  for (uint32_t base = 0; base < total; base += THREADS * UNROLL) {
     V16 v[UNROLL];
+    typename M::cptr spos[UNROLL];
     typename M::ptr dpos[UNROLL];
-    int32_t len[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      len[u] = 0;
-      if (i0 + u * THREADS < total) generic_load<M, WIDE>(c, src, dst, fill, row, slot, &v[u], &dpos[u], &len[u]);
+      const bool inside = base + tid + u * THREADS < total;
+      generic_slot<M>(c, src, dst, fill, inside ? row : rows - 1, inside ? slot : slots - 1, &spos[u], &dpos[u]);
       row += step_rows;
       slot += step_slots;
       if (slot >= slots) {
@@ -248,14 +218,55 @@ MMR_HD void generic_rows(const mmr_copy_chunk& c, typename M::cptr src, typename
       }
     }
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) generic_store<M, WIDE>(dpos[u], len[u], v[u]);
+    for (int u = 0; u < UNROLL; ++u) v[u] = fill ? V16{0, 0, 0, 0} : M::load16u(spos[u]);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) M::template storeu<V16>(dpos[u], v[u]);
+  }
+}
+
+// Rows narrower than 16 bytes: one (row, slot) pair per lane and step, 8/4/2/1-byte pieces.
+template <class M>
+MMR_HD void generic_narrow_load(const mmr_copy_chunk& c, typename M::cptr src, typename M::ptr dst, bool fill, uint32_t row,
+                                uint32_t slot, V16* v, typename M::ptr* dpos, int32_t* len) {
+  typename M::ptr drow = dst + row * c.d1;
+  typename M::cptr srow = src + row * c.s1;
+  const int32_t w = static_cast<int32_t>(c.w);
+  const int32_t mis = static_cast<int32_t>((fill ? M::addr(drow) : M::caddr(srow)) & 15u);
+  const int32_t rel = static_cast<int32_t>(slot << 4) - mis;  // row-relative byte where this aligned slot starts
+  const int32_t lo = rel < 0 ? 0 : rel;
+  const int32_t hi = rel + 16 < w ? rel + 16 : w;
+  *len = hi - lo;
+  *dpos = drow + lo;
+  if (*len > 0) *v = fill ? V16{0, 0, 0, 0} : load_ragged<M>(srow + lo, static_cast<uint32_t>(*len));
+}
+
+template <class M, int THREADS, int UNROLL>
+MMR_HD void generic_narrow_rows(const mmr_copy_chunk& c, typename M::cptr src, typename M::ptr dst, uint32_t tid) {
+  const bool fill = c.src_slot == MMR_SLOT_FILL;
+  const uint32_t slots = 2;  // a row of under 16 bytes touches at most two aligned slots
+  const uint32_t total = c.n1 * slots;
+  for (uint32_t i0 = tid; i0 < total; i0 += THREADS * UNROLL) {
+    V16 v[UNROLL];
+    typename M::ptr dpos[UNROLL];
+    int32_t len[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      len[u] = 0;
+      const uint32_t i = i0 + u * THREADS;
+      if (i < total) generic_narrow_load<M>(c, src, dst, fill, i >> 1, i & 1u, &v[u], &dpos[u], &len[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+      if (len[u] > 0) store_ragged<M>(dpos[u], static_cast<uint32_t>(len[u]), v[u]);
   }
 }
 
 template <class M, int THREADS, int UNROLL>
 MMR_HD void generic_chunk(const mmr_copy_chunk& c, typename M::cptr src, typename M::ptr dst, uint32_t tid) {
-  if (c.w >= 16) generic_rows<M, THREADS, UNROLL, true>(c, src, dst, tid);  // uniform over the workgroup
-  else generic_rows<M, THREADS, UNROLL, false>(c, src, dst, tid);
+  // all three choices are uniform over the workgroup
+  if (c.w < 16) generic_narrow_rows<M, THREADS, UNROLL>(c, src, dst, tid);
+  else if (c.src_slot == MMR_SLOT_FILL) generic_wide_rows<M, THREADS, UNROLL, true>(c, src, dst, tid);
+  else generic_wide_rows<M, THREADS, UNROLL, false>(c, src, dst, tid);
 }
 
 // ---------------------------------------------------------------------------

@@ -77,6 +77,14 @@ __device__ __forceinline__ gchar* slot_base(void* const* __restrict__ ptrs, uint
   return (gchar*)(static_cast<char*>(ptrs[slot])) + off;
 }
 
+// Launch shape of the aligned kernel (overridable at build time for tuning runs).
+#ifndef MMR_COPY16_UNROLL
+#define MMR_COPY16_UNROLL 2
+#endif
+#ifndef MMR_COPY16_NT_LOADS
+#define MMR_COPY16_NT_LOADS true
+#endif
+
 template <int THREADS, int UNROLL>
 __global__ __launch_bounds__(THREADS) void mmr_copy16_kernel(const mmr_copy_chunk* __restrict__ chunks, uint32_t n,
                                                              void* const* __restrict__ ptrs, uint32_t xcd_group) {
@@ -85,7 +93,7 @@ __global__ __launch_bounds__(THREADS) void mmr_copy16_kernel(const mmr_copy_chun
   const mmr_copy_chunk c = chunks[ci];
   gchar* dst = slot_base(ptrs, c.dst_slot, c.dst_off);
   gcchar* src = c.src_slot == MMR_SLOT_FILL ? dst : slot_base(ptrs, c.src_slot, c.src_off);  // never read when filling
-  copy16_chunk<DeviceMem<true, true>, THREADS, UNROLL>(c, src, dst, threadIdx.x);
+  copy16_chunk<DeviceMem<MMR_COPY16_NT_LOADS, true>, THREADS, UNROLL>(c, src, dst, threadIdx.x);
 }
 
 template <int THREADS, int UNROLL, bool NTL, bool NTS>
@@ -254,7 +262,7 @@ hipError_t launch_copy16(const mmr_copy_chunk* d_chunks, int64_t n, void* const*
   if (n == 0) return hipSuccess;
   if (hipError_t e = check_grid(n)) return e;
   const uint32_t group = xcd_group_of(n, xcd_mode);
-  hipLaunchKernelGGL((mmr_copy16_kernel<256, 8>), dim3(grid_size(n, group)), dim3(256), 0, stream, d_chunks,
+  hipLaunchKernelGGL((mmr_copy16_kernel<256, MMR_COPY16_UNROLL>), dim3(grid_size(n, group)), dim3(256), 0, stream, d_chunks,
                      static_cast<uint32_t>(n), d_ptrs, group);
   return hipGetLastError();
 }

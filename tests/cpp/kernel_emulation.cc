@@ -174,8 +174,8 @@ int mmr_emulate_plan(const mmr_plan* plan, void* const* slot_ptrs, const size_t*
         switch (shape) {
           case 1: run_copy16<128, 4>(c, src, dst); break;
           case 2: run_copy16<64, 8>(c, src, dst); break;
-          case 3: run_copy16<512, 2>(c, src, dst); break;
-          default: run_copy16<256, 8>(c, src, dst); break;
+          case 3: run_copy16<512, 1>(c, src, dst); break;
+          default: run_copy16<256, 2>(c, src, dst); break;
         }
       } else {
         if (c.n2 != 1) g_error = "generic chunk with n2 != 1";
