@@ -738,8 +738,9 @@ MMR_HD void transpose_thin_store(const mmr_transpose_chunk& c, typename M::ptr d
   }
 }
 
-// Phase 1 / phase 2 of batch entry b for thread tid, whatever its sub-tile needs.  `wave` = tid / kGroupThreads (the
-// kernel passes it as a wave-uniform value so the choice of path is a scalar branch).
+// Phase 1 / phase 2 of batch entry b for thread tid, whatever its sub-tile needs; `wave` = tid / kGroupThreads.
+// This is how the host emulation walks a chunk.  The kernel makes the same choice once per chunk and wave and then
+// runs a batch loop of its own for the chosen path (see transpose_tiles in kernels.hip for why).
 template <class M, typename T>
 MMR_HD void transpose_load_any(const mmr_transpose_chunk& c, typename M::cptr src, uint32_t b, T* lds, uint32_t tid,
                                uint32_t wave) {
