@@ -170,6 +170,19 @@ class Builder {
     }
     BoxDim dim1 = outer[i1];
     int64_t n1 = std::min(dim1.n, rows);
+    if (aligned && n1 < dim1.n && (dim1.d == w || dim1.s == w)) {
+      // Rows that abut on one side, cut into several chunks along this dim: keep the cuts on 128-byte lines of that
+      // side where a few rows less achieve it, so no line is shared by two workgroups (832-byte rows: 8 per chunk
+      // instead of 9 measured +3 %).
+      int64_t g = w, h = 128;
+      while (h != 0) {
+        const int64_t t = g % h;
+        g = h;
+        h = t;
+      }
+      const int64_t m = 128 / g;
+      if (n1 > m) n1 = n1 / m * m;
+    }
     BoxDim dim2{1, 0, 0};
     int64_t n2 = 1;
     int i2 = -1;
