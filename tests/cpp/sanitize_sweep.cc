@@ -121,8 +121,8 @@ int run_case(std::mt19937_64& rng, int index) {
   std::vector<int64_t> sizes(rank);
   int64_t total = 1;
   for (int i = 0; i < rank; ++i) {
-    const int64_t pool[] = {1, 2, 3, 5, 7, 8, 13, 16, 17, 31, 33, 64, 70, 129};
-    sizes[i] = pool[rng() % 14];
+    const int64_t pool[] = {1, 2, 3, 5, 7, 8, 13, 16, 17, 31, 33, 64, 70, 129, 257, 1030};
+    sizes[i] = pool[rng() % 16];
     if (total * sizes[i] > 60000) sizes[i] = 1 + rng() % 4;
     total *= sizes[i];
   }
