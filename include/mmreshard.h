@@ -146,6 +146,18 @@ int mmr_to_mpmd_sharding(int32_t rank, const mmr_op_sharding* sharding, int64_t 
 /* Shard geometry: what spmd::MakePartitionedShape + ByteSizeOfElements give the
  * plugin (mm_pjrt_executable.cc:537, mm_pjrt_buffer.cc:285-288) and what the
  * mock calls zuku::ShardSize (mm_mock_mm_xla.cc:75). */
+/* ReplicateDims (mm_sharding.cc:458-582; used by sharding propagation, off the reshard path): the tiling of the
+ * given tile-assignment dims moves into the trailing replication dim.  The result's iota is in XLA's canonical
+ * form; the order of devices inside a replication group is not significant (HloSharding sorts each group). */
+int mmr_replicate_dims(const mmr_op_sharding* sharding, const int64_t* replicated_dims, int32_t n_replicated,
+                       mmr_op_sharding* out);
+/* ResizeSharding (mm_sharding.cc:98-161): grows or shrinks the first tiled dim that can take it so that the tile
+ * assignment has num_elements tiles.  *found = 0 where the reference returns nullopt.  dev_count = 0: no device
+ * list given.  devices_out backs out->tile_assignment_devices when the input has an explicit device list. */
+int mmr_resize_sharding(const int64_t* shape, int32_t rank, const mmr_op_sharding* sharding, int64_t num_elements,
+                        int64_t dev_start, int64_t dev_count, mmr_op_sharding* out, int64_t* devices_out,
+                        int64_t devices_capacity, int32_t* found);
+
 int mmr_validate_sharded_shape(const mmr_sharded_shape* s);
 int mmr_shard_extents(const mmr_sharded_shape* s, int64_t* extents, int32_t* rank);
 int mmr_shard_bytes(const mmr_sharded_shape* s, int64_t* bytes);

@@ -8,7 +8,8 @@ from . import _binding
 from ._binding import LIB_PATH, MmrError, load  # noqa: F401
 from .api import (  # noqa: F401
     CanonicalizeSharding, ComputeGlobalIndex, ComputeIndexSet, DeviceListOfSharding, LogicalShardingToOpSharding, LogicalToPhysicalSharding,
-    MeshEquivalentSharding, NeedsReshard, Plan, ReshardContext, StoreHandle, TileAssignmentDevices, ToMpmdSharding,
+    MeshEquivalentSharding, NeedsReshard, Plan, ReplicateDims, ReshardContext, ResizeSharding, StoreHandle, TileAssignmentDevices,
+    ToMpmdSharding,
     XlaShapeToZukuShape, describe, device_of_tile, itemsize, op_sharding, partition_spec_to_sharded_shape, shard_bytes,
     shard_extents,
     sharded_shape, tile_of_device,

@@ -117,6 +117,8 @@ PROTOTYPES = {
     "mmr_needs_reshard": (C.c_int, [I64, I64, I64, I64, P(OpSharding), P(OpSharding), P(I32)]),
     "mmr_device_list_of_sharding": (C.c_int, [P(OpSharding), P(I64), P(I64)]),
     "mmr_to_mpmd_sharding": (C.c_int, [I32, P(OpSharding), I64, I64, I64, I64, P(OpSharding), P(I64), I64]),
+    "mmr_replicate_dims": (C.c_int, [P(OpSharding), P(I64), I32, P(OpSharding)]),
+    "mmr_resize_sharding": (C.c_int, [P(I64), I32, P(OpSharding), I64, I64, I64, P(OpSharding), P(I64), I64, P(I32)]),
     "mmr_validate_sharded_shape": (C.c_int, [P(ShardedShape)]),
     "mmr_shard_extents": (C.c_int, [P(ShardedShape), P(I64), P(I32)]),
     "mmr_shard_bytes": (C.c_int, [P(ShardedShape), P(I64)]),

@@ -201,6 +201,31 @@ def ToMpmdSharding(rank: int, sharding: B.OpSharding, task_devices: Tuple[int, i
     return out
 
 
+def ReplicateDims(replicated_dims: Sequence[int], sharding: B.OpSharding) -> B.OpSharding:
+    """The tiling of the given tile-assignment dims moves into the trailing replication dim
+    (mm_sharding.cc:458-582)."""
+    out = B.OpSharding()
+    B.check(B.load().mmr_replicate_dims(C.byref(sharding), _i64(list(replicated_dims) or [0]), len(replicated_dims),
+                                        C.byref(out)))
+    return out
+
+
+def ResizeSharding(shape: Sequence[int], sharding: B.OpSharding, num_elements: int,
+                   devices: Optional[Tuple[int, int]] = None) -> Optional[B.OpSharding]:
+    """A sharding with `num_elements` tiles grown or shrunk from `sharding`, or None where the reference finds
+    none (mm_sharding.cc:98-161).  `devices` = (start, count)."""
+    out = B.OpSharding()
+    found = C.c_int32()
+    start, count = devices if devices is not None else (0, 0)
+    backing = _i64([0] * max(count, 1))
+    B.check(B.load().mmr_resize_sharding(_i64(list(shape) or [0]), len(shape), C.byref(sharding), num_elements, start, count,
+                                         C.byref(out), backing, max(count, 1), C.byref(found)))
+    if not found.value:
+        return None
+    out._keepalive = backing
+    return out
+
+
 def shard_extents(s: B.ShardedShape) -> Tuple[int, ...]:
     ext = _i64([0] * B.MMR_MAX_DIMS)
     rank = C.c_int32()

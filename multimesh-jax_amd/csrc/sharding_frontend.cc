@@ -43,9 +43,8 @@ int check_sharding(const mmr_op_sharding* s) {
 // walks (HloSharding::FromProto builds every assignment through it): size-1
 // iota dims are dropped and iota dims that stay adjacent and in order after the
 // transpose are merged.
-void canonical_iota(const mmr_op_sharding& s, std::vector<int64_t>* dims, std::vector<int>* perm) {
-  std::vector<int64_t> d(s.iota_reshape_dims, s.iota_reshape_dims + s.n_iota_dims);
-  std::vector<int> p(s.iota_transpose_perm, s.iota_transpose_perm + s.n_iota_dims);
+void canonical_iota(const std::vector<int64_t>& d, const std::vector<int>& p, std::vector<int64_t>* dims,
+                    std::vector<int>* perm) {
   std::vector<int> renum(d.size(), -1);
   std::vector<int64_t> kept;
   for (size_t i = 0; i < d.size(); ++i)
@@ -79,6 +78,11 @@ void canonical_iota(const mmr_op_sharding& s, std::vector<int64_t>* dims, std::v
   }
   perm->clear();
   for (size_t g = 0; g < groups.size(); ++g) perm->push_back(new_index[g]);
+}
+
+void canonical_iota(const mmr_op_sharding& s, std::vector<int64_t>* dims, std::vector<int>* perm) {
+  canonical_iota(std::vector<int64_t>(s.iota_reshape_dims, s.iota_reshape_dims + s.n_iota_dims),
+                 std::vector<int>(s.iota_transpose_perm, s.iota_transpose_perm + s.n_iota_dims), dims, perm);
 }
 
 int map_type(int32_t dtype) {
@@ -494,6 +498,146 @@ int mmr_to_mpmd_sharding(int32_t rank, const mmr_op_sharding* sharding, int64_t 
     r.replicate_on_last_tile_dim = 1;
   }
   *out = r;
+  return MMR_OK;
+}
+
+int mmr_replicate_dims(const mmr_op_sharding* sharding, const int64_t* replicated_dims, int32_t n_replicated,
+                       mmr_op_sharding* out) {
+  if (int rc = check_sharding(sharding)) return rc;
+  if (!out || n_replicated < 0 || (n_replicated > 0 && !replicated_dims)) return fail(MMR_INVALID_ARGUMENT, "null argument");
+  if (sharding->n_iota_dims <= 0)  // mm_sharding.cc:465-468
+    return fail(MMR_INVALID_ARGUMENT, "ReplicateDims only supported for iota tile assignment");
+  const int n_ta = sharding->n_tile_dims;
+  const int64_t* ta = sharding->tile_dims;
+  for (int i = 0; i < n_replicated; ++i)
+    if (replicated_dims[i] < 0 || replicated_dims[i] >= n_ta)
+      return fail(MMR_INVALID_ARGUMENT, "replicated dim %lld of %d tile dims", (long long)replicated_dims[i], n_ta);
+  std::vector<int64_t> reshape;
+  std::vector<int> perm;
+  canonical_iota(*sharding, &reshape, &perm);
+  // :476-514  un-group the iota dims into tile-assignment dims, then order the groups as the transpose does
+  std::vector<std::vector<int>> groups(1);
+  size_t iota_dim = 0;
+  int64_t spanned = 1;
+  int ta_dim = 0;
+  for (; ta_dim < n_ta && iota_dim < perm.size(); ++ta_dim) {
+    spanned *= ta[ta_dim];
+    const int64_t span = reshape[static_cast<size_t>(perm[iota_dim])];
+    groups.back().push_back(ta_dim);
+    if (spanned >= span) {
+      ++iota_dim;
+      if (iota_dim < perm.size()) groups.emplace_back();
+      spanned = 1;
+    }
+  }
+  for (; ta_dim < n_ta; ++ta_dim) groups.back().push_back(ta_dim);
+  if (groups.size() != perm.size()) return fail(MMR_INVALID_ARGUMENT, "iota dims do not group into tile assignment dims");
+  std::vector<int> current;
+  for (int src : perm)
+    for (int d : groups[static_cast<size_t>(src)]) current.push_back(d);
+  // :516-540
+  std::vector<int64_t> new_reshape;
+  for (int d : current) new_reshape.push_back(ta[d]);
+  for (int i = 0; i < n_replicated; ++i) new_reshape.push_back(1);
+  const bool repl_last = sharding->replicate_on_last_tile_dim != 0;
+  const int num_shape_dims = repl_last ? n_ta - 1 : n_ta;
+  std::vector<int> new_perm(current);
+  int extra = static_cast<int>(new_perm.size());
+  for (int i = 0; i < n_replicated; ++i) {
+    const size_t dim = static_cast<size_t>(replicated_dims[i]);
+    if (dim >= current.size()) return fail(MMR_INVALID_ARGUMENT, "replicated dim outside the permutation");
+    new_perm.push_back(current[dim]);
+    new_perm[dim] = extra++;
+  }
+  int64_t total = repl_last ? ta[num_shape_dims] : 1, elements = 1;  // :542-552
+  for (int i = 0; i < n_replicated; ++i) total *= ta[replicated_dims[i]];
+  for (int i = 0; i < n_ta; ++i) elements *= ta[i];
+  mmr_op_sharding r{};
+  if (total == elements) {  // :554-557
+    r.type = MMR_SHARDING_REPLICATED;
+    *out = r;
+    return MMR_OK;
+  }
+  std::vector<int64_t> ta_dims(ta, ta + n_ta);  // :559-571
+  if (repl_last) ta_dims[static_cast<size_t>(num_shape_dims)] = total;
+  else ta_dims.push_back(total);
+  for (int i = 0; i < n_replicated; ++i) ta_dims[static_cast<size_t>(replicated_dims[i])] = 1;
+  // The reference hands the raw lists to HloSharding::FromProto, which keeps the canonical iota; so does this.
+  std::vector<int64_t> cd;
+  std::vector<int> cp;
+  canonical_iota(new_reshape, new_perm, &cd, &cp);
+  if (ta_dims.size() > MMR_MAX_DIMS || cd.size() > MMR_MAX_DIMS)
+    return fail(MMR_UNSUPPORTED, "more than %d tile or iota dims", MMR_MAX_DIMS);
+  r.type = MMR_SHARDING_OTHER;
+  r.n_tile_dims = static_cast<int32_t>(ta_dims.size());
+  for (size_t i = 0; i < ta_dims.size(); ++i) r.tile_dims[i] = ta_dims[i];
+  r.n_iota_dims = static_cast<int32_t>(cd.size());
+  for (size_t i = 0; i < cd.size(); ++i) {
+    r.iota_reshape_dims[i] = cd[i];
+    r.iota_transpose_perm[i] = cp[i];
+  }
+  r.replicate_on_last_tile_dim = 1;
+  r.iota_offset = sharding->iota_offset;
+  *out = r;
+  return MMR_OK;
+}
+
+int mmr_resize_sharding(const int64_t* shape, int32_t rank, const mmr_op_sharding* sharding, int64_t num_elements,
+                        int64_t dev_start, int64_t dev_count, mmr_op_sharding* out, int64_t* devices_out,
+                        int64_t devices_capacity, int32_t* found) {
+  if (int rc = check_sharding(sharding)) return rc;
+  if (!out || !found || (rank > 0 && !shape)) return fail(MMR_INVALID_ARGUMENT, "null argument");
+  *found = 0;
+  const int n_ta = sharding->n_tile_dims;
+  if (n_ta > rank) return fail(MMR_INVALID_ARGUMENT, "%d tile dims for a shape of rank %d", n_ta, rank);
+  if (num_elements < 1) return fail(MMR_INVALID_ARGUMENT, "%lld tiles", (long long)num_elements);
+  const bool has_devices = dev_count > 0;
+  const bool iota = sharding->n_iota_dims > 0;
+  if (iota) {  // mm_sharding.cc:101-109  no answer under a transposed device order
+    std::vector<int64_t> d;
+    std::vector<int> p;
+    canonical_iota(*sharding, &d, &p);
+    for (size_t i = 0; i < p.size(); ++i)
+      if (p[i] != static_cast<int>(i)) return MMR_OK;
+  }
+  int64_t src_size = 1;
+  for (int i = 0; i < n_ta; ++i) src_size *= sharding->tile_dims[i];
+  const int64_t dst_size = num_elements;
+  mmr_op_sharding r{};
+  r.type = MMR_SHARDING_OTHER;
+  bool matched = false;
+  for (int dim = 0; dim < n_ta; ++dim) {  // :120-142
+    const int64_t old_size = sharding->tile_dims[dim];
+    const int64_t new_size = old_size * dst_size / src_size;
+    if (!matched && old_size > 1 && new_size > 0 && new_size <= shape[dim]) {
+      if ((src_size > dst_size && src_size % dst_size) || (src_size < dst_size && dst_size % src_size)) continue;
+      r.tile_dims[r.n_tile_dims++] = new_size;
+      matched = true;
+    } else {
+      r.tile_dims[r.n_tile_dims++] = old_size;
+    }
+    // the reference indexes the dims written so far by `dim`; after a skipped dim that entry does not exist
+    if (dim == n_ta - 1 && sharding->replicate_on_last_tile_dim && r.n_tile_dims == dim + 1 && r.tile_dims[dim] > 1)
+      r.replicate_on_last_tile_dim = 1;
+  }
+  if (!matched) return MMR_OK;
+  int64_t tiles = 1;
+  for (int i = 0; i < r.n_tile_dims; ++i) tiles *= r.tile_dims[i];
+  if (iota || !has_devices) {  // :144-150
+    r.n_iota_dims = 1;
+    r.iota_reshape_dims[0] = num_elements;
+    r.iota_transpose_perm[0] = 0;
+    if (has_devices) r.iota_offset = dev_start;
+    if (tiles != num_elements) return MMR_OK;  // HloSharding::FromProto refuses it
+  } else {  // :151-154
+    if (tiles != dev_count) return MMR_OK;
+    if (!devices_out || devices_capacity < dev_count) return fail(MMR_INVALID_ARGUMENT, "device list output too small");
+    for (int64_t i = 0; i < dev_count; ++i) devices_out[i] = dev_start + i;
+    r.tile_assignment_devices = devices_out;
+    r.n_devices = dev_count;
+  }
+  *out = r;
+  *found = 1;
   return MMR_OK;
 }
 

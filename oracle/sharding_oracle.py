@@ -28,6 +28,12 @@ tests, re-expressed as numbers in tests/golden/sharding_golden.json:
       src/pjrt_client/mpmd_partition.cc:128-166
       pinned by the store shardings mpmd_partition_test.cc:1381-1418 and
       :1455-1484 expect (rebased iota offsets; replication on a submesh)
+  replicate_dims / resize_sharding (same file, off the reshard path: they
+  serve sharding propagation at compile time)
+      src/pjrt_client/mm_sharding.cc:458-582, 98-161
+      pinned by mm_sharding_test.cc:247-527 (9 ReplicateDims cases, compared
+      as tile dims + device order + the replication flag, which is what
+      HloSharding equality compares) and :230-245 (3 ResizeSharding answers)
   canonicalize_sharding
       src/pjrt_client/mm_sharding.cc:275-456
       pinned by mm_sharding_test.cc:529-737 (3 golden descriptors, 1 error)
@@ -461,4 +467,106 @@ def to_mpmd_sharding(rank: int, sharding: OpSharding, task_devices: Tuple[int, i
             if not 0 <= rel < t_count:
                 raise ShardingError("relative device id %d outside the task's %d devices" % (rel, t_count))
         out.tile_assignment_devices = [t_start + rel for rel in sharding.tile_assignment_devices]
+    return out
+
+
+def replicate_dims(replicated_dims: Sequence[int], sharding: OpSharding) -> OpSharding:
+    """mm_sharding.cc:458-582.  Moves the tiling of `replicated_dims` (tile-assignment dims) into the trailing
+    replication dim.  The reference walks the HloSharding's iota, i.e. XLA's canonical form of it."""
+    if not sharding.has_iota:                                                               # :465-468
+        raise ShardingError("ReplicateDims only supported for iota tile assignment")
+    ta = list(sharding.tile_assignment_dimensions)
+    reshape, perm = canonical_iota(sharding.iota_reshape_dims, sharding.iota_transpose_perm)
+    # :476-514  un-group the iota dims into tile-assignment dims, then order the groups as the transpose does
+    groups: List[List[int]] = [[]]
+    iota_dim, spanned, ta_dim = 0, 1, 0
+    while ta_dim < len(ta) and iota_dim < len(perm):
+        spanned *= ta[ta_dim]
+        span = reshape[perm[iota_dim]]
+        groups[-1].append(ta_dim)
+        if spanned >= span:
+            iota_dim += 1
+            if iota_dim < len(perm):
+                groups.append([])
+            spanned = 1
+        ta_dim += 1
+    groups[-1].extend(range(ta_dim, len(ta)))
+    if len(groups) != len(perm):
+        raise ShardingError("iota dims do not group into tile assignment dims")
+    current = [d for src in perm for d in groups[src]]
+    # :516-540
+    new_reshape = [ta[d] for d in current] + [1] * len(replicated_dims)
+    num_shape_dims = len(ta) - 1 if sharding.replicate_on_last_tile_dim else len(ta)
+    new_perm = list(current)
+    extra = len(new_perm)
+    for dim in replicated_dims:
+        new_perm.append(current[dim])
+        new_perm[dim] = extra
+        extra += 1
+    total = ta[num_shape_dims] if sharding.replicate_on_last_tile_dim else 1               # :542-552
+    for dim in replicated_dims:
+        total *= ta[dim]
+    n = 1
+    for d in ta:
+        n *= d
+    if total == n:                                                                          # :554-557
+        return OpSharding(type="REPLICATED")
+    ta_dims = list(ta)                                                                      # :559-571
+    if sharding.replicate_on_last_tile_dim:
+        ta_dims[num_shape_dims] = total
+    else:
+        ta_dims.append(total)
+    for dim in replicated_dims:
+        ta_dims[dim] = 1
+    return OpSharding(type="OTHER", tile_assignment_dimensions=ta_dims, iota_reshape_dims=new_reshape,
+                      iota_transpose_perm=new_perm, replicate_on_last_tile_dim=True,
+                      iota_offset=sharding.iota_offset)
+
+
+def resize_sharding(shape_dims: Sequence[int], sharding: OpSharding, num_elements: int,
+                    devices: Optional[Tuple[int, int]] = None) -> Optional[OpSharding]:
+    """mm_sharding.cc:98-161.  Grows or shrinks the first tiled dim that can take it so that the tile assignment
+    has `num_elements` tiles; None where the reference returns nullopt.  `devices` = (start, count) or None."""
+    if sharding.has_iota:                                                                   # :101-109
+        _, perm = canonical_iota(sharding.iota_reshape_dims, sharding.iota_transpose_perm)
+        if any(i != p for i, p in enumerate(perm)):
+            return None
+    ta = list(sharding.tile_assignment_dimensions)
+    src_size = 1
+    for d in ta:
+        src_size *= d
+    dst_size = num_elements
+    dims: List[int] = []
+    replicate_last = False
+    matched = False
+    for dim, old in enumerate(ta):                                                          # :120-142
+        new = old * dst_size // src_size
+        if not matched and old > 1 and new > 0 and new <= shape_dims[dim]:
+            if (src_size > dst_size and src_size % dst_size) or (src_size < dst_size and dst_size % src_size):
+                continue
+            dims.append(new)
+            matched = True
+        else:
+            dims.append(old)
+        # (the reference indexes the dims written so far by `dim`; after a skipped dim no match can follow, since the
+        # divisibility test that skips does not depend on the dim, and the result is nullopt either way)
+        if dim == len(ta) - 1 and sharding.replicate_on_last_tile_dim and len(dims) == dim + 1 and dims[dim] > 1:
+            replicate_last = True
+    if not matched:
+        return None
+    out = OpSharding(type="OTHER", tile_assignment_dimensions=dims, replicate_on_last_tile_dim=replicate_last)
+    if sharding.has_iota or devices is None:                                                # :144-150
+        out.iota_reshape_dims = [num_elements]
+        out.iota_transpose_perm = [0]
+        if devices is not None:
+            out.iota_offset = devices[0]
+    else:                                                                                   # :151-154
+        out.tile_assignment_devices = list(range(devices[0], devices[0] + devices[1]))
+    # HloSharding::FromProto (XLA) refuses a tile assignment whose tile count differs from its device count
+    n = 1
+    for d in dims:
+        n *= d
+    count = num_elements if out.has_iota else len(out.tile_assignment_devices)
+    if n != count:
+        return None
     return out

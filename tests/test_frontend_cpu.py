@@ -315,6 +315,87 @@ def test_to_mpmd_sharding_known_answers_of_the_reference(golden):
             assert got[k] == e[k], (c["source"], k)
 
 
+def _tiles_up_to_replica_order(devices, tile_dims, replicated_last):
+    """Device ids per tile; inside a replication group the order is not significant (an HloSharding built with
+    replicate_on_last_tile_dim keeps each group sorted, so the reference's EXPECT_EQ compares them that way)."""
+    a = np.asarray(list(devices), dtype=np.int64).reshape(list(tile_dims))
+    return np.sort(a, axis=-1) if replicated_last else a
+
+
+def test_replicate_dims_known_answers_of_the_reference(golden):
+    """mm_sharding_test.cc:247-527: nine ReplicateDims cases (plain, several dims, non-contiguous dims, 4-d, already
+    replicated on the last tile dim, transposed device orders), for the oracle restatement and the C ABI."""
+    cases = golden["replicate_dims"]
+    assert len(cases) == 9
+    for c in cases:
+        e = _oracle_op2(c["expect"])
+        want = _tiles_up_to_replica_order(so.iota_tile_assignment(e).reshape(-1), e.tile_assignment_dimensions, True)
+        o = so.replicate_dims(c["replicated_dims"], _oracle_op2(c["input"]))
+        assert o.tile_assignment_dimensions == e.tile_assignment_dimensions and o.replicate_on_last_tile_dim, c["source"]
+        assert (_tiles_up_to_replica_order(so.iota_tile_assignment(o).reshape(-1), o.tile_assignment_dimensions, True)
+                == want).all(), c["source"]
+        got = mm.ReplicateDims(c["replicated_dims"], _lib_op2(c["input"]))
+        d = _op_dict(got)
+        assert d["tile_dims"] == e.tile_assignment_dimensions and d["replicate_on_last_tile_dim"], c["source"]
+        assert (_tiles_up_to_replica_order(mm.TileAssignmentDevices(got), d["tile_dims"], True) == want).all(), c["source"]
+
+
+def test_replicate_dims_special_cases():
+    """Replicating every tiled dim gives plain replication (mm_sharding.cc:554-557); an explicit device list is
+    refused (:465-468); the tiles of the untouched dims keep their devices' order."""
+    full = mm.op_sharding("OTHER", [2, 4], [8], [0])
+    assert _op_dict(mm.ReplicateDims([0, 1], full))["type"] == "REPLICATED"
+    assert so.replicate_dims([0, 1], so.OpSharding(type="OTHER", tile_assignment_dimensions=[2, 4], iota_reshape_dims=[8],
+                                                   iota_transpose_perm=[0])).type == "REPLICATED"
+    with pytest.raises(mm.MmrError):
+        mm.ReplicateDims([0], mm.op_sharding("OTHER", [2, 1], tile_assignment_devices=[0, 1]))
+    with pytest.raises(so.ShardingError):
+        so.replicate_dims([0], so.OpSharding(type="OTHER", tile_assignment_dimensions=[2, 1], tile_assignment_devices=[0, 1]))
+    # brute force: tile (i, j) of a [3, 5] iota holds device i * 5 + j; replicating dim 0 leaves tile j holding {j, 5 + j, 10 + j}
+    out = mm.ReplicateDims([0], mm.op_sharding("OTHER", [3, 5], [15], [0]))
+    tiles = _tiles_up_to_replica_order(mm.TileAssignmentDevices(out), _op_dict(out)["tile_dims"], True)
+    assert tiles.shape == (1, 5, 3)
+    for j in range(5):
+        assert list(tiles[0, j]) == [j, 5 + j, 10 + j]
+
+
+def test_resize_sharding_known_answers_of_the_reference(golden):
+    """mm_sharding_test.cc:230-248: a 4-way tiling shrinks to 2 tiles, has no answer for 5, and a [2,1,2] tiling of
+    f32[2,8,8] grown to 16 tiles never exceeds the shape's extents."""
+    cases = golden["resize_sharding"]
+    assert len(cases) == 3
+    for c in cases:
+        o = so.resize_sharding(c["shape"], _oracle_op2(c["input"]), c["num_elements"])
+        got = mm.ResizeSharding(c["shape"], _lib_op2(c["input"]), c["num_elements"])
+        assert (o is not None) == c["expect_value"] == (got is not None), c["source"]
+        if not c["expect_value"]:
+            continue
+        d = _op_dict(got)
+        assert d["tile_dims"] == o.tile_assignment_dimensions, c["source"]
+        assert int(np.prod(d["tile_dims"])) == c["num_elements"], c["source"]
+        if "expect_tile_dims" in c:
+            assert d["tile_dims"] == c["expect_tile_dims"], c["source"]
+        if "expect_tile_dims_at_most" in c:
+            assert all(t <= m for t, m in zip(d["tile_dims"], c["expect_tile_dims_at_most"])), c["source"]
+        assert list(mm.TileAssignmentDevices(got)) == list(range(c["num_elements"])), c["source"]
+
+
+def test_resize_sharding_branches():
+    """A transposed device order has no answer (mm_sharding.cc:101-109); with a device list the result starts at its
+    first device (:147-149); an explicit device list in, an explicit consecutive one out (:151-154)."""
+    transposed = mm.op_sharding("OTHER", [2, 2], [2, 2], [1, 0])
+    assert mm.ResizeSharding([8, 8], transposed, 8) is None
+    assert so.resize_sharding([8, 8], so.OpSharding(type="OTHER", tile_assignment_dimensions=[2, 2],
+                                                    iota_reshape_dims=[2, 2], iota_transpose_perm=[1, 0]), 8) is None
+    grown = mm.ResizeSharding([8, 8], mm.op_sharding("OTHER", [2, 1], [2], [0]), 4, (6, 4))
+    assert _op_dict(grown)["tile_dims"] == [4, 1] and list(mm.TileAssignmentDevices(grown)) == [6, 7, 8, 9]
+    listed = mm.ResizeSharding([8, 8], mm.op_sharding("OTHER", [2, 1], tile_assignment_devices=[0, 1]), 4, (6, 4))
+    assert _op_dict(listed)["tile_dims"] == [4, 1] and list(mm.TileAssignmentDevices(listed)) == [6, 7, 8, 9]
+    o = so.resize_sharding([8, 8], so.OpSharding(type="OTHER", tile_assignment_dimensions=[2, 1],
+                                                 tile_assignment_devices=[0, 1]), 4, (6, 4))
+    assert o.tile_assignment_dimensions == [4, 1] and o.tile_assignment_devices == [6, 7, 8, 9]
+
+
 def test_to_mpmd_sharding_special_cases():
     """The branches no reference test exercises, from what they must mean: replication over the whole machine stays
     replication; on a single device the array lives on that device; relative device ids become global ones."""
