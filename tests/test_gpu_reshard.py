@@ -108,9 +108,11 @@ def test_config4_full_size_round_trip_and_samples(ctx):
         ctx.Free(st)
 
 
-def _random_array(rnd, types=("U8", "BF16", "F32", "F64", "C128")):
+def _random_array(rnd, types=("U8", "BF16", "F32", "F64", "C128"), extents=None):
     rank = rnd.randint(1, 4)
-    shape = [rnd.choice([1, 2, 3, 5, 8, 17, 33, 64, 130]) for _ in range(rank)]
+    shape = [rnd.choice(extents or [1, 2, 3, 5, 8, 17, 33, 64, 130]) for _ in range(rank)]
+    while int(np.prod(shape)) > 3_000_000:
+        shape[rnd.randrange(rank)] = rnd.choice([1, 2, 3, 5, 8])
     type_ = rnd.choice(types)
 
     def side(start):
@@ -140,9 +142,10 @@ def test_random_sharding_pairs(ctx):
     permuted layouts (copy, generic and transpose kernels), every element size."""
     rnd = random.Random(1234)
     rng = np.random.Generator(np.random.PCG64(99))
-    for case in range(60):
-        a = _random_array(rnd)
-        say("random case %d: %s %s src=%s dst=%s" % (case, a["type"], a["shape"], a["src"], a["dst"]))
+    for case in range(1500):
+        a = _random_array(rnd, extents=(1, 2, 3, 5, 6, 8, 17, 33, 64, 70, 129, 130, 257, 300, 1030) if case >= 60 else None)
+        if case < 60 or case % 100 == 0:
+            say("random case %d: %s %s src=%s dst=%s" % (case, a["type"], a["shape"], a["src"], a["dst"]))
         item = ro.ITEMSIZE[a["type"]]
         g = rng.integers(0, 256, size=int(np.prod(a["shape"])) * item, dtype=np.uint8).view(
             ro.raw_dtype(a["type"])).reshape(a["shape"])
