@@ -373,10 +373,10 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
   chunk_bytes = std::min<uint32_t>(std::max<uint32_t>(chunk_bytes, 256), 16u << 20) & ~255u;
   plan->options = options;
   // Ragged rows cost more instructions per byte, so their chunks are half the aligned size when a size is asked
-  // for.  By default 7 KiB (8 rows of configuration 5's 820-byte rows), measured best both on configuration 5
-  // (45 MB: 5.40 TB/s against 5.35 at 5.5 KiB, 4.96 at 4 KiB and 5.27 at 7.5 KiB) and on an 8 times larger instance
-  // (5.13 TB/s against 5.00 at 5.5 KiB); a small plan gets smaller chunks so that it still has thousands of them
-  // to spread over 256 CUs.
+  // for.  By default 7 KiB (8 rows of configuration 5's 820-byte rows), measured best on large arrays (360 MB of
+  // them: 5.13 TB/s against 5.00 at 5.5 KiB); a plan under ~58 MB gets proportionally smaller chunks, so that it
+  // still has some 8,000 of them to spread over 256 CUs (configuration 5, 45 MB, buffers not in the Infinity Cache:
+  // 4.35 TB/s at 5 KiB against 4.23 at 7 KiB and 3.95 at 8 KiB).
   uint32_t generic_chunk_bytes = std::max<uint32_t>(chunk_bytes / 2, 256);
   if (options.chunk_bytes == 0) {
     int64_t payload = 0;
@@ -385,7 +385,7 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
       for (int i = 0; i < srcs[a].ndims && i < MMR_MAX_DIMS; ++i) bytes *= std::max<int64_t>(srcs[a].dims[i].size, 1);
       payload += bytes;
     }
-    generic_chunk_bytes = static_cast<uint32_t>(std::min<int64_t>(std::max<int64_t>(payload / 4096, 2048), 7168)) & ~255u;
+    generic_chunk_bytes = static_cast<uint32_t>(std::min<int64_t>(std::max<int64_t>(payload / 8192, 2048), 7168)) & ~255u;
   }
   Builder builder(plan, chunk_bytes, generic_chunk_bytes, (options.flags & MMR_PLAN_ALL_GENERIC) != 0);
   struct SlotInfo {

@@ -187,5 +187,9 @@ def test_generic_chunks_are_bounded_in_lane_work_as_well_as_in_bytes():
     assert plan.stats["n_fill_chunks"] == len(fills)
     fp8_pad = fills[fills["w"] == 1]  # 11008 rows x 1 byte after the 819 valid bytes of the last tile
     assert int(fp8_pad["n1"].sum()) == 11008 and fp8_pad["n1"].max() <= 384
-    # whole rows of 820 bytes come eight to a chunk (7 KiB)
-    assert int(g[g["w"] == 820]["n1"].max()) == 8
+    # whole rows of 820 bytes: 6 to a chunk at this plan's size (45 MB -> ~5.4 KiB chunks), 8 (7 KiB) on a plan 8 times larger
+    assert int(g[g["w"] == 820]["n1"].max()) == 6
+    big = workloads.config(10)
+    plan_big = mm.Plan([lib_shape(a["type"], a["src"]) for a in big], [lib_shape(a["type"], a["dst"]) for a in big])
+    gb = plan_big.copy_chunks(1)
+    assert int(gb[gb["w"] == 820]["n1"].max()) == 8
