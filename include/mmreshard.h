@@ -340,6 +340,17 @@ int mmr_reshard_bind(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const*
  * (mm_pjrt_executable.cc:616-658) for a single mmr_reshard_batch report a bad call where it is made. */
 int mmr_reshard_validate(mmr_context* ctx, mmr_store* src, mmr_store* dst);
 
+/* No counterpart in the reference.  For callers that cannot allocate device memory where they reshard: code that
+ * runs under HIP graph capture, tight serving loops, harnesses that forbid allocation.  Does what mmr_reshard_batch does,
+ * with the same kernels, but the chunk tables and the table of shard pointers of the launch live in a static device
+ * array of MMR_STATIC_SCRATCH_BYTES per GPU instead of allocated memory: the call plans on the host, copies the tables
+ * into that array on the context's stream (through a pinned staging buffer the context has held since its creation)
+ * and launches; it calls no hipMalloc / hipFree.  A plan whose tables exceed the array is refused with MMR_INVALID_ARGUMENT (use mmr_reshard_batch).  Every
+ * call on a GPU shares that GPU's array: calls are safe one after the other on one stream, calls that overlap on one GPU
+ * (two contexts, two streams) race.  No table order tuning. */
+#define MMR_STATIC_SCRATCH_BYTES (8u << 20)
+int mmr_reshard_batch_static(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int32_t n);
+
 /* Build and upload the plan of n descriptor pairs (one batch) ahead of the first
  * reshard, i.e. when the schedule entry is created (MpmdScheduler::AddReshardTask,
  * mpmd_partition.cc:340-351) rather than when it first executes. */

@@ -11,6 +11,7 @@ import os
 MMR_MAX_DIMS = 9
 MMR_SLOT_FILL = 0xFFFFFFFF
 MMR_STORE_FROM_CACHE = 1
+MMR_STATIC_SCRATCH_BYTES = 8 << 20
 
 STATUS_NAMES = {0: "OK", 1: "INVALID_ARGUMENT", 2: "UNSUPPORTED", 3: "OUT_OF_MEMORY",
                 4: "HIP_ERROR", 5: "NOT_FOUND", 6: "INTERNAL"}
@@ -153,6 +154,7 @@ PROTOTYPES = {
     "mmr_store_id": (I64, [VP]),
     "mmr_reshard": (C.c_int, [VP, VP, VP]),
     "mmr_reshard_batch": (C.c_int, [VP, P(VP), P(VP), I32]),
+    "mmr_reshard_batch_static": (C.c_int, [VP, P(VP), P(VP), I32]),
     "mmr_reshard_bind": (C.c_int, [VP, P(VP), P(VP), I32]),
     "mmr_reshard_validate": (C.c_int, [VP, VP, VP]),
     "mmr_sync": (C.c_int, [VP]),

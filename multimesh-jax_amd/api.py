@@ -468,6 +468,16 @@ class ReshardContext:
             self._batch_args = cached = (key, sa, da)
         B.check(self._lib.mmr_reshard_batch(self._h, cached[1], cached[2], n))
 
+    def ReshardBatchStatic(self, srcs: Sequence[StoreHandle], dsts: Sequence[StoreHandle]) -> None:
+        """ReshardBatch without any device allocation: the launch's tables live in the GPU's static scratch array
+        (B.MMR_STATIC_SCRATCH_BYTES); a plan that does not fit raises INVALID_ARGUMENT."""
+        n = len(srcs)
+        if n != len(dsts):
+            raise ValueError("as many destinations as sources")
+        sa = (C.c_void_p * max(n, 1))(*[s._h for s in srcs])
+        da = (C.c_void_p * max(n, 1))(*[d._h for d in dsts])
+        B.check(self._lib.mmr_reshard_batch_static(self._h, sa, da, n))
+
     def Sync(self) -> None:
         B.check(self._lib.mmr_sync(self._h))
 

@@ -30,16 +30,17 @@ constexpr size_t kTileAlign = 4096;
 
 std::atomic<int64_t> g_next_store_id{0};  // NextStoreId, zuku_execute_context_impl.cc:86-89
 
+struct TransposeRun {
+  uint32_t itemsize;
+  bool vector_only;  // every chunk of the run satisfies transpose_is_vector
+  int64_t begin, count;
+};
+
 struct DevicePlan {
   mmr_plan plan;
   mmr_copy_chunk* d_copy16 = nullptr;
   mmr_copy_chunk* d_generic = nullptr;
   mmr_transpose_chunk* d_transposes = nullptr;
-  struct TransposeRun {
-    uint32_t itemsize;
-    bool vector_only;  // every chunk of the run satisfies transpose_is_vector
-    int64_t begin, count;
-  };
   std::vector<TransposeRun> transpose_runs;  // the table is sorted by (itemsize, kind); one launch per run
   bool tuned = false;                        // the table order has been chosen (timed or fixed by the options)
 
@@ -96,6 +97,13 @@ struct mmr_context {
   std::unordered_map<std::string, std::vector<CachedBuffer>> buffer_cache;        // ArrayCache: by descriptor
   std::unordered_map<int64_t, std::unique_ptr<mmr_store>> stores;
   mmr_context_stats stats{};
+  // mmr_reshard_batch_static: this GPU's static scratch array, a pinned staging buffer of the same size and the event
+  // that tells when the last copy out of the staging buffer is done; host-side plans (no device tables) by key
+  char* static_scratch = nullptr;
+  char* static_staging = nullptr;
+  hipEvent_t static_copied = nullptr;
+  bool static_copy_pending = false;
+  std::unordered_map<std::string, std::unique_ptr<mmr_plan>> static_plans;
 };
 
 namespace {
@@ -140,12 +148,10 @@ void drop_bindings_of(mmr_context* ctx, int64_t store_id) {
   }
 }
 
-// Plans n descriptor pairs under `options` and uploads the tables (not cached here).
-int make_device_plan(mmr_context* ctx, const std::vector<mmr_sharded_shape>& srcs, const std::vector<mmr_sharded_shape>& dsts,
-                     const mmr_plan_options& options, DevicePlan* dp) {
-  const int n = static_cast<int>(srcs.size());
-  if (int rc = mmr::build_plan(srcs.data(), dsts.data(), n, options, &dp->plan)) return rc;
-  const std::vector<mmr_transpose_chunk>& tr = dp->plan.transposes;
+// The transpose kernel's LDS tile and lane mapping assume bounds the planner keeps; checked before every first
+// launch of a plan.  Also splits the table into runs of equal element width and kind, one launch each.
+int check_transposes(const mmr_plan& plan, std::vector<TransposeRun>* runs) {
+  const std::vector<mmr_transpose_chunk>& tr = plan.transposes;
   for (const mmr_transpose_chunk& c : tr) {  // the kernel's LDS tile and lane mapping assume these bounds
     uint32_t tile_x = 0, tile_y = 0;
     mmr::transpose_tile_extent(c.itemsize, &tile_x, &tile_y);
@@ -163,10 +169,19 @@ int make_device_plan(mmr_context* ctx, const std::vector<mmr_sharded_shape>& src
   }
   for (int64_t i = 0; i < static_cast<int64_t>(tr.size()); ++i) {
     const bool vec = mmr::transpose_is_vector(tr[i]);
-    if (i == 0 || tr[i].itemsize != tr[i - 1].itemsize || vec != dp->transpose_runs.back().vector_only)
-      dp->transpose_runs.push_back({tr[i].itemsize, vec, i, 0});
-    dp->transpose_runs.back().count += 1;
+    if (i == 0 || tr[i].itemsize != tr[i - 1].itemsize || vec != runs->back().vector_only)
+      runs->push_back({tr[i].itemsize, vec, i, 0});
+    runs->back().count += 1;
   }
+  return MMR_OK;
+}
+
+// Plans n descriptor pairs under `options` and uploads the tables (not cached here).
+int make_device_plan(mmr_context* ctx, const std::vector<mmr_sharded_shape>& srcs, const std::vector<mmr_sharded_shape>& dsts,
+                     const mmr_plan_options& options, DevicePlan* dp) {
+  const int n = static_cast<int>(srcs.size());
+  if (int rc = mmr::build_plan(srcs.data(), dsts.data(), n, options, &dp->plan)) return rc;
+  if (int rc = check_transposes(dp->plan, &dp->transpose_runs)) return rc;
   if (int rc = upload(ctx, dp->plan.copy16, &dp->d_copy16)) return rc;
   if (int rc = upload(ctx, dp->plan.generic, &dp->d_generic)) return rc;
   if (int rc = upload(ctx, dp->plan.transposes, &dp->d_transposes)) return rc;
@@ -191,21 +206,24 @@ int get_plan(mmr_context* ctx, const std::vector<mmr_sharded_shape>& srcs, const
   return MMR_OK;
 }
 
-// One launch per kernel class over the plan's tables.
-int launch_plan(mmr_context* ctx, const DevicePlan* dp, void* const* d_ptrs) {
-  const mmr_plan& p = dp->plan;
+// One launch per kernel class over the tables of plan `p` as they lie in device memory.
+int launch_tables(mmr_context* ctx, const mmr_plan& p, const mmr_copy_chunk* d_copy16, const mmr_copy_chunk* d_generic,
+                  const mmr_transpose_chunk* d_transposes, const std::vector<TransposeRun>& runs, void* const* d_ptrs) {
   const uint32_t xm = p.options.xcd_mode;
   // aligned chunks: runs of 64 table neighbours per XCD measured best across the benchmark configurations
-  MMR_HIP(mmr::launch_copy16(dp->d_copy16, static_cast<int64_t>(p.copy16.size()), d_ptrs, xm == 0 ? 64 : xm, ctx->stream));
+  MMR_HIP(mmr::launch_copy16(d_copy16, static_cast<int64_t>(p.copy16.size()), d_ptrs, xm == 0 ? 64 : xm, ctx->stream));
   // generic chunks leave partial lines at run boundaries and share source lines with the chunks of neighbouring
   // destination tiles; table neighbours merge both when they share an L2: runs of 64 per XCD (measured)
-  MMR_HIP(mmr::launch_copy_generic(dp->d_generic, static_cast<int64_t>(p.generic.size()), d_ptrs, xm == 0 ? 64 : xm,
-                                   ctx->stream));
-  for (const DevicePlan::TransposeRun& run : dp->transpose_runs)
+  MMR_HIP(mmr::launch_copy_generic(d_generic, static_cast<int64_t>(p.generic.size()), d_ptrs, xm == 0 ? 64 : xm, ctx->stream));
+  for (const TransposeRun& run : runs)
     // tiles are ordered in 8 x 8 blocks; runs of 64 table neighbours per XCD keep a block in one L2 (measured best)
-    MMR_HIP(mmr::launch_transpose(dp->d_transposes + run.begin, run.count, d_ptrs, xm == 0 ? 64 : xm, run.itemsize,
+    MMR_HIP(mmr::launch_transpose(d_transposes + run.begin, run.count, d_ptrs, xm == 0 ? 64 : xm, run.itemsize,
                                   run.vector_only, ctx->stream));
   return MMR_OK;
+}
+
+int launch_plan(mmr_context* ctx, const DevicePlan* dp, void* const* d_ptrs) {
+  return launch_tables(ctx, dp->plan, dp->d_copy16, dp->d_generic, dp->d_transposes, dp->transpose_runs, d_ptrs);
 }
 
 int64_t launches_of(const DevicePlan* dp) {
@@ -288,11 +306,8 @@ int check_store(mmr_context* ctx, const mmr_store* s, const char* what) {
   return MMR_OK;
 }
 
-int reshard_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int n, bool launch = true) {
-  if (n == 0) return MMR_OK;
-  if (int rc = use_device(ctx)) return rc;
-  std::vector<int64_t> ids;
-  ids.reserve(2 * n);
+// Argument checks shared by every reshard entry point.
+int check_batch(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int n) {
   for (int a = 0; a < n; ++a) {
     if (int rc = check_store(ctx, srcs[a], "source")) return rc;
     if (int rc = check_store(ctx, dsts[a], "destination")) return rc;
@@ -301,14 +316,23 @@ int reshard_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* d
     if (srcs[a]->offloaded() || dsts[a]->offloaded())
       return fail(MMR_INVALID_ARGUMENT, "array %d: store %lld is still offloaded to host memory", a,
                   (long long)(srcs[a]->offloaded() ? srcs[a]->id : dsts[a]->id));
-    ids.push_back(srcs[a]->id);
   }
-  for (int a = 0; a < n; ++a) ids.push_back(dsts[a]->id);
   for (int a = 0; a < n; ++a)
     for (int b = 0; b < n; ++b)
       if (dsts[a] == srcs[b] || (a != b && dsts[a] == dsts[b]))
         return fail(MMR_INVALID_ARGUMENT, "store %lld is written by array %d and used again by array %d of the same batch",
                     (long long)dsts[a]->id, a, b);
+  return MMR_OK;
+}
+
+int reshard_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int n, bool launch = true) {
+  if (n == 0) return MMR_OK;
+  if (int rc = use_device(ctx)) return rc;
+  if (int rc = check_batch(ctx, srcs, dsts, n)) return rc;
+  std::vector<int64_t> ids;
+  ids.reserve(2 * n);
+  for (int a = 0; a < n; ++a) ids.push_back(srcs[a]->id);
+  for (int a = 0; a < n; ++a) ids.push_back(dsts[a]->id);
 
   if (launch) ctx->stats.reshard_calls += 1;
   Binding* binding = nullptr;
@@ -362,6 +386,69 @@ int reshard_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* d
   return MMR_OK;
 }
 
+// mmr_reshard_batch_static: the same argument checks, plan and kernels as reshard_locked, but the tables of the launch
+// go into this GPU's static scratch array (host plan -> pinned staging -> one stream-ordered copy) and nothing is
+// allocated on the device.  Layout in the array: pointer table, then the three chunk tables, each 256-byte aligned.
+int reshard_static_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int n) {
+  if (n == 0) return MMR_OK;
+  if (int rc = use_device(ctx)) return rc;
+  if (int rc = check_batch(ctx, srcs, dsts, n)) return rc;
+  std::vector<mmr_sharded_shape> sshapes(n), dshapes(n);
+  for (int a = 0; a < n; ++a) {
+    sshapes[a] = srcs[a]->shape;
+    dshapes[a] = dsts[a]->shape;
+  }
+  std::string key = mmr::plan_key(sshapes.data(), dshapes.data(), n, ctx->options);
+  auto it = ctx->static_plans.find(key);
+  if (it == ctx->static_plans.end()) {
+    auto plan = std::make_unique<mmr_plan>();
+    if (int rc = mmr::build_plan(sshapes.data(), dshapes.data(), n, ctx->options, plan.get())) return rc;
+    it = ctx->static_plans.emplace(std::move(key), std::move(plan)).first;
+  }
+  const mmr_plan& p = *it->second;
+  std::vector<TransposeRun> runs;
+  if (int rc = check_transposes(p, &runs)) return rc;
+  auto round_up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
+  const size_t ptr_bytes = static_cast<size_t>(p.n_slots) * sizeof(void*);
+  const size_t off16 = round_up(ptr_bytes);
+  const size_t off_generic = off16 + round_up(p.copy16.size() * sizeof(mmr_copy_chunk));
+  const size_t off_transposes = off_generic + round_up(p.generic.size() * sizeof(mmr_copy_chunk));
+  const size_t total = off_transposes + round_up(p.transposes.size() * sizeof(mmr_transpose_chunk));
+  if (total > MMR_STATIC_SCRATCH_BYTES)
+    return fail(MMR_INVALID_ARGUMENT,
+                "the tables of this reshard take %zu bytes, the static scratch array holds %u: use mmr_reshard_batch", total,
+                static_cast<unsigned>(MMR_STATIC_SCRATCH_BYTES));
+  if (ctx->static_copy_pending) {  // the staging buffer is free again once the previous call's copy has read it
+    MMR_HIP(hipEventSynchronize(ctx->static_copied));
+    ctx->static_copy_pending = false;
+  }
+  void** ptrs = reinterpret_cast<void**>(ctx->static_staging);
+  for (int a = 0; a < n; ++a) {
+    size_t slot = static_cast<size_t>(p.slot_bases[a]);
+    for (int64_t k = 0; k < srcs[a]->side.dev_count; ++k) ptrs[slot++] = srcs[a]->tile(k);
+    for (int64_t k = 0; k < dsts[a]->side.dev_count; ++k) ptrs[slot++] = dsts[a]->tile(k);
+  }
+  if (!p.copy16.empty()) std::memcpy(ctx->static_staging + off16, p.copy16.data(), p.copy16.size() * sizeof(mmr_copy_chunk));
+  if (!p.generic.empty())
+    std::memcpy(ctx->static_staging + off_generic, p.generic.data(), p.generic.size() * sizeof(mmr_copy_chunk));
+  if (!p.transposes.empty())
+    std::memcpy(ctx->static_staging + off_transposes, p.transposes.data(), p.transposes.size() * sizeof(mmr_transpose_chunk));
+  // stream-ordered: the copy waits for the kernels of the previous call on this stream, which still read the array
+  MMR_HIP(hipMemcpyAsync(ctx->static_scratch, ctx->static_staging, total, hipMemcpyHostToDevice, ctx->stream));
+  MMR_HIP(hipEventRecord(ctx->static_copied, ctx->stream));
+  ctx->static_copy_pending = true;
+  ctx->stats.reshard_calls += 1;
+  char* base = ctx->static_scratch;
+  const int64_t launches = static_cast<int64_t>(runs.size()) + (p.copy16.empty() ? 0 : 1) + (p.generic.empty() ? 0 : 1);
+  if (int rc = launch_tables(ctx, p, reinterpret_cast<const mmr_copy_chunk*>(base + off16),
+                             reinterpret_cast<const mmr_copy_chunk*>(base + off_generic),
+                             reinterpret_cast<const mmr_transpose_chunk*>(base + off_transposes), runs,
+                             reinterpret_cast<void* const*>(base)))
+    return rc;
+  ctx->stats.kernel_launches += launches;
+  return MMR_OK;
+}
+
 int tile_index(const mmr_store* s, int64_t device, int64_t* k) {
   const int64_t rel = device - s->side.dev_start;
   if (rel < 0 || rel >= s->side.dev_count)
@@ -394,6 +481,10 @@ int mmr_context_create(int32_t hip_device, void* hip_stream, mmr_context** out) 
   }
   MMR_HIP(hipEventCreate(&ctx->t0));
   MMR_HIP(hipEventCreate(&ctx->t1));
+  // set-up of the entry point that may not allocate: everything it needs exists from here on
+  MMR_HIP(mmr::static_scratch_address(hip_device, reinterpret_cast<void**>(&ctx->static_scratch)));
+  MMR_HIP(hipHostMalloc(reinterpret_cast<void**>(&ctx->static_staging), MMR_STATIC_SCRATCH_BYTES, hipHostMallocDefault));
+  MMR_HIP(hipEventCreateWithFlags(&ctx->static_copied, hipEventDisableTiming));
   *out = ctx.release();
   return MMR_OK;
 }
@@ -412,6 +503,8 @@ void mmr_context_destroy(mmr_context* ctx) {
     for (auto& b : c.second) (void)hipFree(b.base);
   (void)hipEventDestroy(ctx->t0);
   (void)hipEventDestroy(ctx->t1);
+  if (ctx->static_copied) (void)hipEventDestroy(ctx->static_copied);
+  if (ctx->static_staging) (void)hipHostFree(ctx->static_staging);
   if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
   delete ctx;
 }
@@ -698,6 +791,12 @@ int mmr_reshard_batch(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const
   if (!ctx || n < 0 || (n > 0 && (!srcs || !dsts))) return fail(MMR_INVALID_ARGUMENT, "bad batch arguments");
   std::lock_guard<std::mutex> lock(ctx->mu);
   return reshard_locked(ctx, srcs, dsts, n);
+}
+
+int mmr_reshard_batch_static(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int32_t n) {
+  if (!ctx || n < 0 || (n > 0 && (!srcs || !dsts))) return fail(MMR_INVALID_ARGUMENT, "bad batch arguments");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  return reshard_static_locked(ctx, srcs, dsts, n);
 }
 
 int mmr_reshard_validate(mmr_context* ctx, mmr_store* src, mmr_store* dst) {

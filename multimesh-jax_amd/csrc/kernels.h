@@ -27,6 +27,10 @@ hipError_t launch_copy_generic(const mmr_copy_chunk* d_chunks, int64_t n, void* 
 hipError_t launch_transpose(const mmr_transpose_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
                             uint32_t itemsize, bool vector_only, hipStream_t stream);
 
+// Device address of this GPU's static scratch array (MMR_STATIC_SCRATCH_BYTES long, 256-byte aligned), looked up once
+// per device; `device` must be the current device of the calling thread.
+hipError_t static_scratch_address(int device, void** out);
+
 }  // namespace mmr
 
 #endif  // MMR_CSRC_KERNELS_H_

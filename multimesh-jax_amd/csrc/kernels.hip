@@ -14,6 +14,7 @@
 
 #include <algorithm>
 #include <cstdint>
+#include <mutex>
 
 #include "chunk_ops.h"
 #include "kernels.h"
@@ -238,6 +239,11 @@ __global__ __launch_bounds__(256) void mmr_flat_copy_kernel(const void* __restri
   }
 }
 
+// Device memory that exists without any allocation call: the tables of a launch issued by callers that may not
+// allocate (the static entry point of the C ABI).  One copy per GPU, held until the process ends.  In host code the
+// array's name is only a handle for hipGetSymbolAddress; the device address it yields is what launches and copies use.
+static __device__ __align__(256) unsigned char scratch[MMR_STATIC_SCRATCH_BYTES];
+
 hipError_t check_grid(int64_t n) { return (n < 0 || n > 0x7ff00000LL) ? hipErrorInvalidValue : hipSuccess; }
 
 }  // namespace
@@ -247,6 +253,25 @@ hipError_t check_grid(int64_t n) { return (n < 0 || n > 0x7ff00000LL) ? hipError
 // accesses in flight per lane before the first store; one workgroup per chunk
 // (persistent workgroups that loop over the table, 4 to 16 per CU, with the
 // next chunk record prefetched, were 2-18 % slower on every configuration).
+hipError_t static_scratch_address(int device, void** out) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mu;
+  static void* address[kMaxDevices] = {};
+  if (!out || device < 0 || device >= kMaxDevices) return hipErrorInvalidValue;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!address[device]) {
+    int current = -1;
+    if (hipError_t e = hipGetDevice(&current)) return e;
+    if (current != device) return hipErrorInvalidDevice;  // every GPU holds its own copy of the array at its own address
+    void* ptr = nullptr;
+    if (hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch))) return e;
+    if (!ptr) return hipErrorInvalidSymbol;
+    address[device] = ptr;
+  }
+  *out = address[device];
+  return hipSuccess;
+}
+
 hipError_t launch_flat_copy(const void* src, void* dst, size_t bytes, hipStream_t stream) {
   if (bytes == 0) return hipSuccess;
   if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst) | bytes) & 15u) return hipErrorInvalidValue;

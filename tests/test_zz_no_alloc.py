@@ -1,0 +1,74 @@
+"""The entry point that allocates nothing (mmr_reshard_batch_static): same kernels as mmr_reshard_batch, tables in
+the GPU's static scratch array.  Checked through the C ABI against mmr_reshard_batch, bit for bit, on two calls in a
+row, the second with a smaller input."""
+import sys
+
+import pytest
+
+import multimesh_jax_amd as mm
+from multimesh_jax_amd import _binding as B, workloads
+
+from gpu_helpers import make_stores, read_all
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print("[gpu-test] " + msg, flush=True)
+    sys.stdout.flush()
+
+
+def _both_ways(ctx, arrays):
+    """Reshards `arrays` through the allocating entry point and through the static one (separate, poison-filled
+    destination stores); returns both sets of destination shards and the device bytes allocated in between."""
+    gs = [workloads.generate(a) for a in arrays]
+    srcs, dsts_ref = make_stores(ctx, arrays, gs)
+    _, dsts_static = make_stores(ctx, arrays, gs)
+    ctx.ReshardBatch(srcs, dsts_ref)
+    ctx.Sync()
+    before = ctx.stats
+    ctx.ReshardBatchStatic(srcs, dsts_static)
+    ctx.Sync()
+    after = ctx.stats
+    ref = [read_all(ctx, d) for d in dsts_ref]
+    got = [read_all(ctx, d) for d in dsts_static]
+    return ref, got, before, after
+
+
+def _assert_equal(arrays, ref, got):
+    for a, r, g in zip(arrays, ref, got):
+        assert sorted(r) == sorted(g)
+        for dev in r:
+            assert g[dev].tobytes() == r[dev].tobytes(), (a["name"], dev)
+
+
+def test_static_entry_point_matches_batch_on_two_calls_in_a_row():
+    with mm.ReshardContext(0) as ctx:
+        # first call: configuration 2 at 1/2 scale (aligned chunks, 16,384 of them) together with the ragged arrays of
+        # configuration 5 at 1/8 scale (generic chunks and pad fills) and a transposed layout (tile chunks)
+        first = workloads.config(2, 2) + workloads.config(5, 8) + workloads.config(13, 8)
+        say("static entry point, first call: %d arrays" % len(first))
+        ref, got, before, after = _both_ways(ctx, first)
+        _assert_equal(first, ref, got)
+        assert after["bytes_allocated"] == before["bytes_allocated"]
+        assert after["plans_built"] == before["plans_built"] and after["bindings_built"] == before["bindings_built"]
+        assert after["kernel_launches"] - before["kernel_launches"] >= 3
+        # second call, smaller: the array still holds the first call's tables beyond what this one overwrites
+        second = workloads.config(5, 16)
+        say("static entry point, second call: %d arrays" % len(second))
+        ref, got, before, after = _both_ways(ctx, second)
+        _assert_equal(second, ref, got)
+        assert after["bytes_allocated"] == before["bytes_allocated"]
+
+
+def test_static_entry_point_refuses_plans_beyond_the_array():
+    with mm.ReshardContext(0) as ctx:
+        arrays = workloads.config(4, 2)  # 195 arrays, ~160k chunks: more than 8 MiB of tables
+        gs = [workloads.generate(a) for a in arrays]
+        srcs, dsts = make_stores(ctx, arrays, gs, poison=None)
+        say("static entry point, oversized plan")
+        with pytest.raises(B.MmrError) as e:
+            ctx.ReshardBatchStatic(srcs, dsts)
+        assert e.value.status_name == "INVALID_ARGUMENT" and "static scratch" in str(e.value)
+        ctx.ReshardBatch(srcs, dsts)  # the allocating entry point takes it
+        ctx.Sync()
