@@ -2,17 +2,28 @@
 """Benchmark of the cross-submesh reshard on one MI355X.
 
 A step is one reshard (one pass of the hot path over one batch of synthetic
-input).  The default workload is configuration 2 of BASELINE.json, the one the
+input).  The headline workload is configuration 2 of BASELINE.json, the one the
 metric is quoted on: a bf16 [8, 4096, 8192] activation resharded from
 hidden-sharded 8 ways (devices 0-7) to sequence-sharded 4 ways (devices 8-11),
 all twelve shard buffers resident in this GPU's HBM before the timed region
-starts.  Prints one JSON line.
+starts.  The other four configurations are measured with the same protocol and
+reported under `all_configs`.  Prints one JSON line.
+
+Protocol (per configuration): every result is first compared bit for bit with
+the oracle; buffer sets are rotated between launches so that the 256 MB
+Infinity Cache serves none of the reads; W warm-up launches; K launches timed
+as a whole (wall clock bracketed by synchronisation -> `value`; HIP events on
+the library's stream around the same K launches -> `roofline.achieved`); then
+at least 50 more launches with a timing mark between each two -> median and
+p10 / p90 per launch.
 
 No torch in this process: PyTorch's wheel bundles its own HIP runtime and two
 HIP runtimes cannot both drive the GPU.  The library owns its stream and its
 device memory, and raises if no GPU is present (there is no CPU fallback).
 """
 import argparse
+import glob
+import hashlib
 import json
 import os
 import sys
@@ -24,6 +35,21 @@ if ROOT not in sys.path:
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
+# FETCH_SIZE reads low by this factor, WRITE_SIZE by none: what the two counters report (KiB) for a 512 MiB device
+# copy of known size, measured with the runtime's own hipMemcpyDtoD kernel and with this library's copy kernel
+FETCH_SCALE, WRITE_SCALE = 1.969, 1.000
+
+
+def kernel_sources_digest():
+    """Digest of the sources the kernels and the planner are built from: a traffic profile measured on other
+    sources says nothing about this build."""
+    h = hashlib.sha256()
+    base = os.path.join(ROOT, "multimesh-jax_amd", "csrc")
+    for name in sorted(os.listdir(base)):
+        if name.endswith((".hip", ".h", ".cc")):
+            with open(os.path.join(base, name), "rb") as f:
+                h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()[:16]
 
 
 def cpu_baseline(arrays, gs, seconds=12.0):
@@ -34,7 +60,10 @@ def cpu_baseline(arrays, gs, seconds=12.0):
     from helpers import oracle_shape, raw_global
     from multimesh_jax_amd import workloads
 
-    threads = min(len(os.sched_getaffinity(0)), int(os.environ.get("OMP_NUM_THREADS", "16") or 16), 64)
+    visible = len(os.sched_getaffinity(0))
+    # the GPU box grants one GPU's share of its host (16 threads; it exports OMP_NUM_THREADS accordingly)
+    share = int(os.environ.get("OMP_NUM_THREADS", "0") or 0)
+    threads = min(visible, share) if share > 0 else visible
     a, g = arrays[0], gs[0]
     so, do = oracle_shape(a["type"], a["src"]), oracle_shape(a["type"], a["dst"])
     shards = ro.make_shards(raw_global(a, g), so, a["src"].get("minor_to_major"))
@@ -55,34 +84,61 @@ def cpu_baseline(arrays, gs, seconds=12.0):
     one, reps1, dt1 = timed(1, seconds * 0.3)
     many, reps, dt = timed(threads, seconds * 0.7)
     return {"value": round(many, 2), "unit": "GB/s", "cores": threads, "kind": "port",
-            "single_thread_value": round(one, 2),
-            "sample": "configuration 2 at full size: %d repetitions in %.1f s on %d pthreads (and %d repetitions in "
-                      "%.1f s on 1 thread); C restatement of the reference reshard, one memcpy per contiguous run"
-                      % (reps, dt, threads, reps1, dt1)}, out
+            "single_thread_value": round(one, 2), "host_cores_visible": visible,
+            "sample": "configuration 2 at full size: %d repetitions in %.1f s on %d pthreads (this box's share of its "
+                      "host: %d hardware threads visible) and %d repetitions in %.1f s on 1 thread; C restatement of the "
+                      "reference reshard, one memcpy per contiguous run"
+                      % (reps, dt, threads, visible, reps1, dt1)}, out
 
 
-def measure(ctx, mm, workloads, args, config, with_parity=True):
-    """Creates the stores of one configuration, checks the result against the
-    oracle, times `args.steps` reshards.  Returns (result dict, arrays, gs, first destination stores)."""
-    from gpu_helpers import make_stores, read_all
+def percentile(sorted_values, q):
+    if not sorted_values:
+        return None
+    i = min(len(sorted_values) - 1, max(0, int(round(q * (len(sorted_values) - 1)))))
+    return sorted_values[i]
+
+
+def check_parity(ctx, arrays, gs, dsts, sample_only):
+    """GPU result against the oracle, bit for bit; for the 10 GB pytree a sample of its arrays (every array of the
+    first layer, the embedding and the output head)."""
+    from gpu_helpers import read_all
     from helpers import oracle_outputs
 
-    arrays = workloads.config(config, args.scale)
+    picked = range(len(arrays))
+    if sample_only:
+        picked = [i for i, a in enumerate(arrays) if a["name"].startswith("layer00.") or "." not in a["name"]]
+    for i in picked:
+        expect = oracle_outputs(arrays[i], gs[i])
+        got = read_all(ctx, dsts[i])
+        for dev in expect:
+            if got[dev].tobytes() != expect[dev].tobytes():
+                sys.exit("bench.py: GPU result differs from the oracle (array %s, device %d)" % (arrays[i]["name"], dev))
+    return len(list(picked))
+
+
+def measure(ctx, mm, workloads, args, config):
+    """Creates the stores of one configuration, checks the result against the oracle, times it.
+    Returns (result dict, arrays, gs, first destination stores, first source stores)."""
+    from gpu_helpers import make_stores
+    from helpers import lib_shape
+
+    arrays = workloads.load_json(args.workload_json) if args.workload_json else workloads.config(config, args.scale)
     if args.name:
         arrays = [a for a in arrays if args.name in a["name"]]
     gs = [workloads.generate(a) for a in arrays]
     alg_bytes = workloads.algorithmic_bytes(arrays)
-    # Buffer sets rotated between steps: at least `--sets`, and enough of them that 768 MiB of other buffers are
+    # Buffer sets rotated between launches: at least `--sets`, and enough of them that 768 MiB of other buffers are
     # touched before a set comes round again - the 256 MB Infinity Cache must not serve a small configuration's reads
     # (an explicit --sets 1 or 2 is a probing run and is taken as given).
     n_sets = max(1, args.sets)
     if args.sets >= 3:
         n_sets = max(n_sets, -(-(768 << 20) // max(alg_bytes, 1)) + 1)
     sets = [make_stores(ctx, arrays, gs, poison=None) for _ in range(n_sets)]
+    single = len(arrays) == 1
 
     def step(i):
         srcs, dsts = sets[i % len(sets)]
-        if len(srcs) == 1:
+        if single:
             ctx.Reshard(srcs[0], dsts[0])
         elif args.unbatched:  # one call and one launch per array, as the reference's schedule loop issues them
             for s_, d_ in zip(srcs, dsts):
@@ -90,23 +146,30 @@ def measure(ctx, mm, workloads, args, config, with_parity=True):
         else:
             ctx.ReshardBatch(srcs, dsts)
 
+    # Schedule-build time work (MpmdScheduler::AddReshardTask in the reference): plan, optional timing of launch
+    # orders on the first set, device tables for every set.  None of it is in the timed region.
     before = ctx.stats
     step(0)
     ctx.Sync()
     launches = ctx.stats["kernel_launches"] - before["kernel_launches"]
-    if with_parity and alg_bytes <= (2 << 30):  # parity before timing: bit for bit against the oracle
-        for a, g, d in zip(arrays, gs, sets[0][1]):
-            expect = oracle_outputs(a, g)
-            got = read_all(ctx, d)
-            for dev in expect:
-                if got[dev].tobytes() != expect[dev].tobytes():
-                    sys.exit("bench.py: GPU result differs from the oracle (array %s, device %d)" % (a["name"], dev))
+    checked = check_parity(ctx, arrays, gs, sets[0][1], sample_only=alg_bytes > (2 << 30))
+    order_used = 0
+    if args.tune and not args.unbatched:
+        order_used = ctx.TuneReshard(sets[0][0], sets[0][1])
+    if not args.unbatched:
+        for srcs, dsts in sets:
+            ctx.BindReshard(srcs, dsts)
+    if args.tune and not args.unbatched:  # whatever order was kept, the bytes are the oracle's
+        step(0)
+        ctx.Sync()
+        check_parity(ctx, arrays, gs, sets[0][1], sample_only=alg_bytes > (2 << 30))
 
     for i in range(args.warmup):
         step(i)
     ctx.Sync()
+    syncs_before = ctx.stats["host_blocking_syncs"]
     # timed region: exactly K steps, wall clock bracketed by synchronisation;
-    # HIP events on the library's own stream give the kernel time inside it
+    # HIP events on the library's own stream give the device time inside it
     t0 = time.perf_counter()
     ctx.StartTimer()
     for i in range(args.steps):
@@ -114,40 +177,110 @@ def measure(ctx, mm, workloads, args, config, with_parity=True):
     kernel_ms = ctx.StopTimer()
     ctx.Sync()
     wall_s = time.perf_counter() - t0
+    syncs_in_region = ctx.stats["host_blocking_syncs"] - syncs_before
+    # per-launch distribution: a timing mark between each two of at least 50 back-to-back launches
+    n_laps = max(50, min(args.steps, 500))
+    ctx.Lap()
+    for i in range(n_laps):
+        step(i)
+        ctx.Lap()
+    laps = sorted(ctx.Laps())
 
-    batched = len(arrays) > 1 and not getattr(args, "unbatched", False)
-    plan = (ctx.plan_stats(sets[0][0][0], sets[0][1][0]) if len(arrays) == 1 else
+    batched = len(arrays) > 1 and not args.unbatched
+    plan = (ctx.plan_stats(sets[0][0][0], sets[0][1][0]) if single else
             ctx.batch_plan_stats(sets[0][0], sets[0][1]) if batched else None)
-    # cold plan construction (host only, excluded from the steady-state figure: plans are cached per descriptor pair)
-    from helpers import lib_shape
+    # cold plan construction (host only, outside the steady-state figure: plans are cached per descriptor pair)
     src_shapes = [lib_shape(a["type"], a["src"]) for a in arrays]
     dst_shapes = [lib_shape(a["type"], a["dst"]) for a in arrays]
     tp = time.perf_counter()
-    cold = mm.Plan(src_shapes, dst_shapes, args.chunk_bytes, args.order, args.xcd_mode)
+    cold = mm.Plan(src_shapes, dst_shapes, args.chunk_bytes, args.order, args.xcd_mode, args.flags)
     plan_build_ms = (time.perf_counter() - tp) * 1e3
     table_bytes = cold.stats["table_bytes"]
     del cold
-    generic = plan is not None and plan["n_copy_generic_chunks"] > plan["n_copy16_chunks"]
+    kernel = "mmr_copy16_kernel"
+    if plan is not None:
+        kinds = [("mmr_transpose_kernel", plan["n_transpose_chunks"] * 32768), ("mmr_span_kernel", plan["n_span_chunks"] * 8192),
+                 ("mmr_copy_generic_kernel", plan["n_copy_generic_chunks"] * 5120), ("mmr_copy16_kernel", plan["n_copy16_chunks"] * 8192)]
+        kernel = max(kinds, key=lambda kv: kv[1])[0]  # the class that moves most of the bytes
+    med = percentile(laps, 0.5)
     res = {
         "alg_bytes": alg_bytes,
         "ms_per_step": wall_s * 1e3 / args.steps,
         "value": alg_bytes / (wall_s / args.steps) / 1e9,
         "kernel_ms": kernel_ms / args.steps,
         "achieved": alg_bytes / (kernel_ms / args.steps * 1e-3) / 1e9,
-        "launches": launches,
-        "plan": plan,
-        "plan_build_ms": plan_build_ms,
-        "plan_table_bytes": table_bytes,
-        "kernel": ("mmr_transpose_kernel" if plan is not None and plan["n_transpose_chunks"] > 0 else
-                   "mmr_copy_generic_kernel" if generic or config in (5, 6) else "mmr_copy16_kernel"),
-        "n_arrays": len(arrays),
-        "sets": len(sets),
+        "median_ms": med, "p10_ms": percentile(laps, 0.1), "p90_ms": percentile(laps, 0.9), "laps": len(laps),
+        "median_gbs": alg_bytes / (med * 1e-3) / 1e9 if med else None,
+        "launches": launches, "plan": plan, "plan_build_ms": plan_build_ms, "plan_table_bytes": table_bytes,
+        "kernel": kernel, "n_arrays": len(arrays), "sets": len(sets), "order_used": order_used,
+        "orders_timed": plan["orders_timed"] if plan else 0, "parity_arrays": checked,
+        "host_blocking_syncs_in_timed_region": syncs_in_region,
     }
     first_dsts = sets[0][1]
     for srcs, dsts in sets[1:]:
         for s in srcs + dsts:
             ctx.Free(s)
     return res, arrays, gs, first_dsts, sets[0][0]
+
+
+def traffic_of(config, args):
+    """HBM bytes per launch of the dominant kernel from the committed counter profile of this configuration
+    (profiles/traffic_config<c>.json, written by --record-traffic from rocprofv3 --pmc runs), or null when that
+    profile was measured on other kernel or planner sources than the ones this build comes from."""
+    path = os.path.join(ROOT, "profiles", "traffic_config%d.json" % config)
+    if not os.path.exists(path) or args.scale != 1 or args.name or args.workload_json:
+        return None, None
+    with open(path) as f:
+        prof = json.load(f)
+    if prof.get("kernel_sources_digest") != kernel_sources_digest():
+        return None, "profiles/traffic_config%d.json is stale: measured on kernel sources %s, these are %s" % (
+            config, prof.get("kernel_sources_digest"), kernel_sources_digest())
+    return prof.get("hbm_bytes_per_launch"), "profiles/traffic_config%d.json (%s)" % (config, prof.get("source", ""))
+
+
+def record_traffic(args):
+    """Writes profiles/traffic_config<c>.json from the two counter runs of one configuration:
+         rocprofv3 --pmc FETCH_SIZE --kernel-trace --output-format csv -d <dir>/FETCH_SIZE -o p -- python3 bench.py --config c ...
+         rocprofv3 --pmc WRITE_SIZE ... -d <dir>/WRITE_SIZE ...
+       (one counter per run).  Counter values are KiB per dispatch."""
+    import csv
+    from multimesh_jax_amd import workloads
+    out = {}
+    kernel = None
+    for counter, scale in (("FETCH_SIZE", FETCH_SCALE), ("WRITE_SIZE", WRITE_SCALE)):
+        files = glob.glob(os.path.join(args.record_traffic, counter, "**", "*counter_collection.csv"), recursive=True)
+        if not files:
+            sys.exit("no counter_collection.csv under %s/%s" % (args.record_traffic, counter))
+        per_kernel = {}
+        with open(files[0]) as f:
+            for row in csv.DictReader(f):
+                if "mmr_" in row["Kernel_Name"] and row["Counter_Name"] == counter:
+                    per_kernel.setdefault(row["Kernel_Name"].split("(")[0], []).append(float(row["Counter_Value"]))
+        name, values = max(per_kernel.items(), key=lambda kv: sum(kv[1]))
+        kernel = name
+        out[counter] = {"kib_mean": sum(values) / len(values), "kib_min": min(values), "kib_max": max(values),
+                        "dispatches": len(values), "scale": scale}
+    alg = workloads.algorithmic_bytes(workloads.config(args.config))
+    hbm = int((out["FETCH_SIZE"]["kib_mean"] * FETCH_SCALE + out["WRITE_SIZE"]["kib_mean"] * WRITE_SCALE) * 1024)
+    prof = {"config": args.config, "kernel": kernel, "counters": out, "hbm_bytes_per_launch": hbm,
+            "algorithmic_bytes": alg, "ratio": round(hbm / alg, 4), "kernel_sources_digest": kernel_sources_digest(),
+            "source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, one counter per run, KiB per dispatch; "
+                      "FETCH_SIZE x %.3f, WRITE_SIZE x %.3f" % (FETCH_SCALE, WRITE_SCALE)}
+    path = os.path.join(ROOT, "profiles", "traffic_config%d.json" % args.config)
+    with open(path, "w") as f:
+        json.dump(prof, f, indent=1)
+        f.write("\n")
+    print(json.dumps(prof))
+
+
+def summary(r):
+    return {"GB/s": round(r["achieved"], 1), "frac_hbm_peak": round(r["achieved"] / HBM_PEAK_GBS, 4),
+            "kernel_ms": round(r["kernel_ms"], 5), "median_ms": round(r["median_ms"], 5),
+            "p10_ms": round(r["p10_ms"], 5), "p90_ms": round(r["p90_ms"], 5), "launches_timed": r["laps"],
+            "median_GB/s": round(r["median_gbs"], 1), "algorithmic_bytes": r["alg_bytes"],
+            "launches_per_step": r["launches"], "kernel": r["kernel"], "buffer_sets": r["sets"],
+            "plan_build_ms_cold": round(r["plan_build_ms"], 3), "plan_table_bytes": r["plan_table_bytes"],
+            "order_used": r["order_used"], "orders_timed": r["orders_timed"], "parity_arrays_checked": r["parity_arrays"]}
 
 
 def main():
@@ -157,10 +290,16 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", type=int, default=2, help="BASELINE.json configuration (1-5); 2 is the headline")
     ap.add_argument("--sets", type=int, default=3, help="independent buffer sets rotated between steps")
-    ap.add_argument("--all", action="store_true", help="also measure configurations 1, 3, 4 and 5 (adds minutes)")
+    ap.add_argument("--only", action="store_true", help="measure --config alone (no all_configs)")
+    ap.add_argument("--all", action="store_true", help="accepted for compatibility: all_configs is the default")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-tune", dest="tune", action="store_false",
+                    help="keep the planner's default launch order instead of timing a few on the first buffer set")
     ap.add_argument("--unbatched", action="store_true",
                     help="multi-array configurations: one Reshard call per array instead of one batched call (probing)")
+    ap.add_argument("--record-traffic", type=str, default="",
+                    help="directory with FETCH_SIZE/ and WRITE_SIZE/ rocprofv3 --pmc outputs of --config: writes "
+                         "profiles/traffic_config<c>.json and exits (needs no GPU)")
     # plan options (0 = library default) and probing switches
     ap.add_argument("--chunk-bytes", type=int, default=0)
     ap.add_argument("--order", type=int, default=0)
@@ -168,10 +307,16 @@ def main():
     ap.add_argument("--flags", type=int, default=0)
     ap.add_argument("--name", type=str, default="", help="only the arrays whose name contains this")
     ap.add_argument("--scale", type=int, default=1, help="divide the large extents (probing only)")
+    ap.add_argument("--workload-json", type=str, default="",
+                    help="measure the arrays described in this JSON file instead of a BASELINE.json configuration "
+                         "(a list of {name, type, shape, src, dst, seed, dist} as multimesh-jax_amd/workloads.py builds them)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: every logical device of both submeshes is a buffer in one "
                  "MI355X's HBM and nothing here uses a second GPU (got --gpus %d)" % args.gpus)
+    if args.record_traffic:
+        record_traffic(args)
+        return
 
     import multimesh_jax_amd as mm
     from multimesh_jax_amd import workloads
@@ -182,12 +327,7 @@ def main():
         ctx.set_plan_options(args.chunk_bytes, args.order, args.xcd_mode, args.flags)
 
     res, arrays, gs, first_dsts, first_srcs = measure(ctx, mm, workloads, args, args.config)
-
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic_config%d.json" % args.config)
-    if os.path.exists(tpath) and args.scale == 1 and not args.name:
-        with open(tpath) as f:
-            traffic = json.load(f).get("hbm_bytes_per_launch")
+    traffic, traffic_source = traffic_of(args.config, args)
 
     result = {
         "metric": "reshard GB/s ((read+write bytes)/time) & % HBM peak, bf16 [8,4096,8192]",
@@ -203,22 +343,26 @@ def main():
         "dtype": "u8",  # pure byte movement (bf16 payload never interpreted), 16-byte vector accesses
         "data": "synthetic",
         "config": {
-            "workload": "configuration %d of BASELINE.json: %s" % (
-                args.config, "; ".join("%s %s %s" % (a["name"], a["type"], list(a["shape"])) for a in arrays[:3])
-                + (" ... (%d arrays)" % len(arrays) if len(arrays) > 3 else "")),
+            "workload": (args.workload_json or "configuration %d of BASELINE.json" % args.config) + ": " + "; ".join(
+                "%s %s %s" % (a["name"], a["type"], list(a["shape"])) for a in arrays[:3])
+                + (" ... (%d arrays)" % len(arrays) if len(arrays) > 3 else ""),
             "source": arrays[0]["src"], "destination": arrays[0]["dst"],
             "algorithmic_bytes": res["alg_bytes"], "buffer_sets": res["sets"],
             "plan": res["plan"], "plan_build_ms_cold": round(res["plan_build_ms"], 3),
             "plan_table_bytes": res["plan_table_bytes"], "pct_hbm_peak": round(100.0 * res["value"] / HBM_PEAK_GBS, 2),
+            "order_used": res["order_used"], "orders_timed": res["orders_timed"],
+            "host_blocking_syncs_in_timed_region": res["host_blocking_syncs_in_timed_region"],
         },
         "roofline": {
             "bound": "hbm", "achieved": round(res["achieved"], 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(res["achieved"] / HBM_PEAK_GBS, 4), "traffic": traffic,
+            "frac": round(res["achieved"] / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
             "kernel": res["kernel"], "kernel_ms": round(res["kernel_ms"], 5),
+            "median_ms": round(res["median_ms"], 5), "p10_ms": round(res["p10_ms"], 5), "p90_ms": round(res["p90_ms"], 5),
+            "launches_timed_one_by_one": res["laps"], "median_GB/s": round(res["median_gbs"], 1),
             "launches_per_step": res["launches"],
         },
     }
-    if not args.no_cpu_baseline and args.config == 2 and args.scale == 1:
+    if not args.no_cpu_baseline and args.config == 2 and args.scale == 1 and not args.workload_json:
         base, cpu_out = cpu_baseline(arrays, gs)
         got = read_all(ctx, first_dsts[0])
         for dev, buf in cpu_out.items():
@@ -229,19 +373,21 @@ def main():
         result["cpu_baseline"] = None
     for s in first_srcs + first_dsts:
         ctx.Free(s)
+    ctx.ClearStoreCache()
 
-    if args.all:
+    if not args.only and not args.workload_json and args.scale == 1 and not args.name:
         others = {}
-        for c in (1, 3, 4, 5):
+        for c in (1, 2, 3, 4, 5):
             if c == args.config:
                 continue
-            r, *_rest = measure(ctx, mm, workloads, args, c)
-            others["config%d" % c] = {"GB/s": round(r["achieved"], 1), "frac_hbm_peak": round(r["achieved"] / HBM_PEAK_GBS, 4),
-                                       "kernel_ms": round(r["kernel_ms"], 5), "algorithmic_bytes": r["alg_bytes"],
-                                       "launches_per_step": r["launches"], "kernel": r["kernel"],
-                                       "plan_build_ms_cold": round(r["plan_build_ms"], 3)}
-            for s in _rest[2] + _rest[3]:
+            r, _arrays, _gs, dsts_, srcs_ = measure(ctx, mm, workloads, args, c)
+            others["config%d" % c] = summary(r)
+            t, tsrc = traffic_of(c, args)
+            others["config%d" % c]["traffic"] = t
+            others["config%d" % c]["traffic_source"] = tsrc
+            for s in srcs_ + dsts_:
                 ctx.Free(s)
+            ctx.ClearStoreCache()
         result["all_configs"] = others
     ctx.close()
     print(json.dumps(result))

@@ -205,8 +205,10 @@ typedef struct {
   int64_t src_bstride, dst_bstride;
 } mmr_transpose_chunk;
 
-#define MMR_PLAN_ALL_GENERIC 1u
-#define MMR_PLAN_NO_AUTOTUNE 2u
+#define MMR_PLAN_ALL_GENERIC 1u /* treat every tile as ragged (aligned boxes go through the span kernel too; testing) */
+#define MMR_PLAN_NO_AUTOTUNE 2u /* accepted and ignored: table orders are only timed on request (mmr_reshard_tune) */
+#define MMR_PLAN_NO_SPAN 4u     /* ragged boxes become generic chunks instead of span groups (testing) */
+#define MMR_PLAN_NO_INLINE 8u   /* group tables always live in device memory, never in the kernel's argument block */
 
 typedef struct {
   uint32_t chunk_bytes; /* target bytes per copy chunk, 0 = default */
@@ -225,7 +227,10 @@ typedef struct {
 typedef struct {
   int64_t n_arrays;
   int64_t n_boxes;             /* source-tile x destination-tile overlaps */
-  int64_t n_copy16_chunks;     /* 16-byte aligned copy chunks */
+  int64_t n_copy16_chunks;     /* 16-byte aligned copy chunks (workgroups of the copy-group launch) */
+  int64_t n_span_chunks;       /* destination spans (workgroups of the span launch, ragged rows) */
+  int64_t n_groups;            /* records of the group tables ... */
+  int64_t n_pieces;            /* ... and their pieces */
   int64_t n_copy_generic_chunks;
   int64_t n_transpose_chunks;
   int64_t n_fill_chunks;       /* included in the two copy counts */
@@ -262,14 +267,28 @@ void mmr_context_destroy(mmr_context* ctx);
 int mmr_context_stream(mmr_context* ctx, void** hip_stream);
 /* Default plan options of the context (chunk size, ordering); affects plans built afterwards. */
 int mmr_context_set_plan_options(mmr_context* ctx, const mmr_plan_options* options);
+/* Checking mode, kept from the reference's mock runtime: a rolling hash of the operation stream (kind, store ids,
+ * descriptors; mm_mock_mm_xla.cc:259-262, compared between runs at mm_pjrt_executable_test.cc:760-766) and, on every
+ * reshard, "every operand holds a tile on each of its devices" (mm_mock_mm_xla.cc:347-369).  Off by default. */
+#define MMR_CHECK_INVARIANTS 1u
+int mmr_context_set_flags(mmr_context* ctx, uint32_t flags);
 
-#define MMR_STORE_FROM_CACHE 1u /* CreateStoreConfig::allocate_from_cache */
+#define MMR_STORE_FROM_CACHE 1u    /* CreateStoreConfig::allocate_from_cache */
+#define MMR_STORE_UNINITIALIZED 2u /* skip the zero fill: for stores whose every byte a reshard writes before it is read
+                                      (a reshard writes the pad of short tiles too) */
 
 /* CreateStore / CreateStoreImpl, zuku_execute_context.h:99-104,
  * zuku_execute_context_impl.cc:521-550: allocates the buffer of every device of
  * the descriptor's device list (zero-filled). */
 int mmr_store_create(mmr_context* ctx, const mmr_sharded_shape* shape, const char* name, uint32_t flags,
                      mmr_store** out);
+/* The same with CreateStoreConfig::min_cache_size (zuku_execute_context.h:29, passed to ArrayCache::Get at
+ * zuku_execute_context_impl.cc:529-535; the mock prints value_or(1), mm_mock_mm_xla.cc:238).  ArrayCache itself is
+ * third-party; read here as: with MMR_STORE_FROM_CACHE, the cache of this descriptor is made to hold at least
+ * min_cache_size buffers in total (the one handed out included), so the next min_cache_size - 1 requests for the
+ * descriptor are served without allocating.  Values < 1 count as 1. */
+int mmr_store_create_ex(mmr_context* ctx, const mmr_sharded_shape* shape, const char* name, uint32_t flags,
+                        int64_t min_cache_size, mmr_store** out);
 /* Zero-copy import (what AssembleShards' "TODO: do the slicing" flat copy,
  * zuku_execute_context_impl.cc:405-415, would become when the native PjRt
  * shards may be used in place): a store whose buffer of device dev_start + k IS
@@ -279,8 +298,13 @@ int mmr_store_adopt(mmr_context* ctx, const mmr_sharded_shape* shape, const char
                     mmr_store** out);
 
 /* OffloadDtoH / OffloadHtoD, zuku_execute_context.h:61-68,
- * zuku_execute_context_impl.cc:162-211: move every buffer of the store to
- * pinned host memory and release the device memory / bring it back.  Blocking.
+ * zuku_execute_context_impl.cc:162-211: the store's buffers move between the
+ * device cache and a host cache of pinned buffers (both keyed by descriptor),
+ * by an asynchronous copy on the context's stream; neither call waits for the
+ * device.  The device memory an offload gives up goes to the device cache (the
+ * next store of that descriptor created with MMR_STORE_FROM_CACHE takes it,
+ * ordered on the stream behind the copy); the pinned buffer a reload gives up
+ * goes to the host cache.  mmr_clear_store_cache releases both.
  * An offloaded store cannot be resharded, assembled or sliced (the mock's
  * invariant, mm_mock_mm_xla.cc:347-356); mmr_store_read_shard still works. */
 int mmr_store_offload(mmr_context* ctx, mmr_store* store);
@@ -288,9 +312,13 @@ int mmr_store_reload(mmr_context* ctx, mmr_store* store);
 int mmr_store_is_offloaded(const mmr_store* store, int32_t* out);
 
 /* Free, zuku_execute_context_impl.cc:504-515 (keep_in_cache: buffers go back to
- * the per-shape cache); Destroy, :356-361. The handle is dead afterwards. */
+ * the per-shape cache); Destroy, :356-361. The handle is dead afterwards.  Without
+ * keep_in_cache the memory returns to the context's allocator pool (the reference
+ * allocates every store through its cache, :533-535): the next store of the same
+ * byte size takes it, so freeing does not wait for the device. */
 int mmr_store_free(mmr_context* ctx, mmr_store* store, int32_t keep_in_cache);
-/* ClearStoreCache, zuku_execute_context_impl.cc:517-519. */
+/* ClearStoreCache, zuku_execute_context_impl.cc:517-519: releases the per-shape cache, the allocator pool and the
+ * pinned host cache. */
 int mmr_clear_store_cache(mmr_context* ctx);
 
 /* AssembleShards / Shard{data, local_device_id, size},
@@ -348,8 +376,19 @@ int mmr_reshard_validate(mmr_context* ctx, mmr_store* src, mmr_store* dst);
  * and launches; it calls no hipMalloc / hipFree.  A plan whose tables exceed the array is refused with MMR_INVALID_ARGUMENT (use mmr_reshard_batch).  Every
  * call on a GPU shares that GPU's array: calls are safe one after the other on one stream, calls that overlap on one GPU
  * (two contexts, two streams) race.  No table order tuning. */
-#define MMR_STATIC_SCRATCH_BYTES (8u << 20)
+#define MMR_STATIC_SCRATCH_BYTES (1u << 20)
 int mmr_reshard_batch_static(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int32_t n);
+
+/* Times a few launch orders of the plan of these stores on the stores themselves (a reshard is idempotent) and keeps
+ * the fastest for every later reshard of the same descriptors; *order_used receives its mmr_plan_options.order value
+ * (0 = the default stayed).  Blocks the calling thread for a few dozen launches.  Nothing else ever times a plan: a
+ * plain mmr_reshard plans, uploads and launches without waiting for the device, and its plan is the same on every
+ * run.  Call it where the schedule is built (MpmdScheduler::AddReshardTask, mpmd_partition.cc:340-351), before any
+ * graph capture of the reshard. */
+int mmr_reshard_tune(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int32_t n, int64_t* order_used);
+/* Drops every cached plan and binding (device tables) no launch in flight needs; pinned ones (mmr_reshard_bind) go
+ * too, so graphs captured from them must not be replayed afterwards.  Waits for the stream. */
+int mmr_context_clear_plans(mmr_context* ctx);
 
 /* Build and upload the plan of n descriptor pairs (one batch) ahead of the first
  * reshard, i.e. when the schedule entry is created (MpmdScheduler::AddReshardTask,
@@ -369,6 +408,11 @@ int mmr_sync(mmr_context* ctx);
  * zuku_execute_context_impl.cc:462-486, measure wall clock; here device time). */
 int mmr_timer_start(mmr_context* ctx);
 int mmr_timer_stop(mmr_context* ctx, float* milliseconds); /* blocks */
+/* Per-launch timing of back-to-back work: mmr_timer_lap records a mark on the stream (between two launches, say);
+ * mmr_timer_laps blocks until the last mark is reached, writes the device time between consecutive marks
+ * (marks - 1 values, at most `capacity`; *count = how many) and forgets the marks. */
+int mmr_timer_lap(mmr_context* ctx);
+int mmr_timer_laps(mmr_context* ctx, float* milliseconds, int32_t capacity, int32_t* count);
 
 typedef struct {
   int64_t plans_built;
@@ -381,8 +425,17 @@ typedef struct {
   int64_t bytes_high_watermark;
   int64_t stores_live;
   int64_t cache_hits;      /* store buffers served from the per-shape cache */
-  int64_t host_bytes_allocated; /* pinned host bytes of offloaded stores */
+  int64_t host_bytes_allocated; /* pinned host bytes of offloaded stores and of the host cache */
   int64_t host_bytes_high_watermark;
+  int64_t host_blocking_syncs;  /* times an entry point made the calling thread wait for the device */
+  int64_t inline_launches;      /* launches whose table travelled in the kernel's argument block */
+  int64_t device_allocations;   /* hipMalloc calls */
+  int64_t host_cache_hits;      /* offloads served from the pinned host cache */
+  int64_t pool_hits;            /* new stores whose memory came from the allocator's pool of freed stores */
+  int64_t plans_cached;         /* plans held now */
+  int64_t bindings_cached;      /* bound device tables held now */
+  int64_t invariant_checks;     /* checks made in MMR_CHECK_INVARIANTS mode */
+  int64_t operation_hash;       /* rolling hash of the operation stream in that mode */
 } mmr_context_stats;
 int mmr_context_get_stats(mmr_context* ctx, mmr_context_stats* out);
 /* Stats of the cached plan of a store pair (builds it if needed). */

@@ -11,7 +11,10 @@ import os
 MMR_MAX_DIMS = 9
 MMR_SLOT_FILL = 0xFFFFFFFF
 MMR_STORE_FROM_CACHE = 1
-MMR_STATIC_SCRATCH_BYTES = 8 << 20
+MMR_STORE_UNINITIALIZED = 2
+MMR_PLAN_ALL_GENERIC, MMR_PLAN_NO_AUTOTUNE, MMR_PLAN_NO_SPAN = 1, 2, 4
+MMR_CHECK_INVARIANTS = 1
+MMR_STATIC_SCRATCH_BYTES = 1 << 20
 
 STATUS_NAMES = {0: "OK", 1: "INVALID_ARGUMENT", 2: "UNSUPPORTED", 3: "OUT_OF_MEMORY",
                 4: "HIP_ERROR", 5: "NOT_FOUND", 6: "INTERNAL"}
@@ -80,7 +83,8 @@ class PlanOptions(C.Structure):
 
 class PlanStats(C.Structure):
     _fields_ = [(n, C.c_int64) for n in (
-        "n_arrays", "n_boxes", "n_copy16_chunks", "n_copy_generic_chunks", "n_transpose_chunks",
+        "n_arrays", "n_boxes", "n_copy16_chunks", "n_span_chunks", "n_groups", "n_pieces", "n_copy_generic_chunks",
+        "n_transpose_chunks",
         "n_fill_chunks", "bytes_moved", "bytes_filled", "table_bytes", "n_slots", "order_used", "interleave_kib",
         "orders_timed")]
 
@@ -92,7 +96,9 @@ class ContextStats(C.Structure):
     _fields_ = [(n, C.c_int64) for n in (
         "plans_built", "plan_cache_hits", "bindings_built", "binding_cache_hits", "kernel_launches",
         "reshard_calls", "bytes_allocated", "bytes_high_watermark", "stores_live", "cache_hits",
-        "host_bytes_allocated", "host_bytes_high_watermark")]
+        "host_bytes_allocated", "host_bytes_high_watermark", "host_blocking_syncs", "inline_launches",
+        "device_allocations", "host_cache_hits", "pool_hits", "plans_cached", "bindings_cached", "invariant_checks",
+        "operation_hash")]
 
     def as_dict(self):
         return {n: getattr(self, n) for n, _ in self._fields_}
@@ -136,6 +142,10 @@ PROTOTYPES = {
     "mmr_context_stream": (C.c_int, [VP, P(VP)]),
     "mmr_context_set_plan_options": (C.c_int, [VP, P(PlanOptions)]),
     "mmr_store_create": (C.c_int, [VP, P(ShardedShape), C.c_char_p, C.c_uint32, P(VP)]),
+    "mmr_store_create_ex": (C.c_int, [VP, P(ShardedShape), C.c_char_p, C.c_uint32, I64, P(VP)]),
+    "mmr_context_set_flags": (C.c_int, [VP, C.c_uint32]),
+    "mmr_context_clear_plans": (C.c_int, [VP]),
+    "mmr_reshard_tune": (C.c_int, [VP, P(VP), P(VP), I32, P(I64)]),
     "mmr_store_adopt": (C.c_int, [VP, P(ShardedShape), C.c_char_p, P(VP), P(VP)]),
     "mmr_store_offload": (C.c_int, [VP, VP]),
     "mmr_store_reload": (C.c_int, [VP, VP]),
@@ -160,6 +170,8 @@ PROTOTYPES = {
     "mmr_sync": (C.c_int, [VP]),
     "mmr_timer_start": (C.c_int, [VP]),
     "mmr_timer_stop": (C.c_int, [VP, P(C.c_float)]),
+    "mmr_timer_lap": (C.c_int, [VP]),
+    "mmr_timer_laps": (C.c_int, [VP, P(C.c_float), I32, P(I32)]),
     "mmr_context_get_stats": (C.c_int, [VP, P(ContextStats)]),
     "mmr_reshard_plan_stats": (C.c_int, [VP, VP, VP, P(PlanStats)]),
     "mmr_reshard_batch_plan_stats": (C.c_int, [VP, P(VP), P(VP), I32, P(PlanStats)]),

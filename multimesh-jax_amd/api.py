@@ -265,12 +265,12 @@ class Plan:
     """Copy plan of one or more (source, destination) descriptor pairs."""
 
     def __init__(self, srcs: Sequence[B.ShardedShape], dsts: Sequence[B.ShardedShape],
-                 chunk_bytes: int = 0, order: int = 0, xcd_mode: int = 0):
+                 chunk_bytes: int = 0, order: int = 0, xcd_mode: int = 0, flags: int = 0):
         if isinstance(srcs, B.ShardedShape):
             srcs, dsts = [srcs], [dsts]
         self._lib = B.load()
         self._h = C.c_void_p()
-        opt = B.PlanOptions(chunk_bytes, order, xcd_mode, 0)
+        opt = B.PlanOptions(chunk_bytes, order, xcd_mode, flags)
         B.check(self._lib.mmr_plan_create(_shape_array(srcs), _shape_array(dsts), len(srcs), C.byref(opt),
                                           C.byref(self._h)))
 
@@ -286,7 +286,8 @@ class Plan:
         return st.as_dict()
 
     def copy_chunks(self, kind: int) -> np.ndarray:
-        """kind 0: 16-byte aligned chunks, kind 1: generic chunks (structured array)."""
+        """kind 0: the chunks of the copy-group launch, decoded in launch order; kind 1: generic chunks;
+        kind 2: the row pieces of the span groups, one record each (structured array)."""
         n = self._lib.mmr_plan_get_copy_chunks(self._h, kind, None, 0)
         buf = (B.CopyChunk * max(n, 1))()
         self._lib.mmr_plan_get_copy_chunks(self._h, kind, buf, n)
@@ -361,11 +362,12 @@ class ReshardContext:
 
     # -- stores -----------------------------------------------------------
     def CreateStore(self, shape: B.ShardedShape, name: Optional[str] = None,
-                    allocate_from_cache: bool = False) -> StoreHandle:
+                    allocate_from_cache: bool = False, min_cache_size: int = 1,
+                    uninitialized: bool = False) -> StoreHandle:
         h = C.c_void_p()
-        flags = B.MMR_STORE_FROM_CACHE if allocate_from_cache else 0
-        B.check(self._lib.mmr_store_create(self._h, C.byref(shape), name.encode() if name else None, flags,
-                                           C.byref(h)))
+        flags = (B.MMR_STORE_FROM_CACHE if allocate_from_cache else 0) | (B.MMR_STORE_UNINITIALIZED if uninitialized else 0)
+        B.check(self._lib.mmr_store_create_ex(self._h, C.byref(shape), name.encode() if name else None, flags,
+                                              min_cache_size, C.byref(h)))
         return StoreHandle(self, h, shape, name or "anonymous")
 
     def AssembleShards(self, shape: B.ShardedShape, device: int, data, existing_store: Optional[StoreHandle] = None,
@@ -419,6 +421,24 @@ class ReshardContext:
         sa = (C.c_void_p * max(n, 1))(*[s._h for s in srcs])
         da = (C.c_void_p * max(n, 1))(*[d._h for d in dsts])
         B.check(self._lib.mmr_reshard_bind(self._h, sa, da, n))
+
+    def TuneReshard(self, srcs, dsts) -> int:
+        """Times a few launch orders of the plan of these stores on the stores themselves and keeps the fastest
+        (blocking; never done implicitly).  Returns the order now in use (0 = the default)."""
+        if isinstance(srcs, StoreHandle):
+            srcs, dsts = [srcs], [dsts]
+        n = len(srcs)
+        sa = (C.c_void_p * max(n, 1))(*[s._h for s in srcs])
+        da = (C.c_void_p * max(n, 1))(*[d._h for d in dsts])
+        used = C.c_int64()
+        B.check(self._lib.mmr_reshard_tune(self._h, sa, da, n, C.byref(used)))
+        return used.value
+
+    def ClearPlans(self) -> None:
+        B.check(self._lib.mmr_context_clear_plans(self._h))
+
+    def set_flags(self, flags: int) -> None:
+        B.check(self._lib.mmr_context_set_flags(self._h, flags))
 
     def SliceLocalShard(self, device: int, store: StoreHandle, wait: bool = True) -> int:
         p = C.c_void_p()
@@ -493,6 +513,17 @@ class ReshardContext:
         ms = C.c_float()
         B.check(self._lib.mmr_timer_stop(self._h, C.byref(ms)))
         return ms.value
+
+    def Lap(self) -> None:
+        """A timing mark on the stream (see Laps)."""
+        B.check(self._lib.mmr_timer_lap(self._h))
+
+    def Laps(self, capacity: int = 4096) -> List[float]:
+        """Device milliseconds between consecutive marks set with Lap() (blocks until the last one is reached)."""
+        buf = (C.c_float * capacity)()
+        n = C.c_int32()
+        B.check(self._lib.mmr_timer_laps(self._h, buf, capacity, C.byref(n)))
+        return [buf[i] for i in range(n.value)]
 
     @property
     def stream(self) -> int:

@@ -43,6 +43,7 @@ constexpr uint32_t kXcds = 8;  // MI355X: 256 CUs in 8 XCDs, each with its own L
 // workgroups map to indices >= n and do nothing.
 MMR_HD uint32_t chunk_index(uint32_t block, uint32_t group) {
   if (group <= 1) return block;
+  if (group == 64) return ((((block >> 9) << 3) + (block & 7u)) << 6) | ((block >> 3) & 63u);  // the usual case, no division
   const uint32_t xcd = block % kXcds, j = block / kXcds;
   return ((j / group) * kXcds + xcd) * group + (j % group);
 }

@@ -10,6 +10,8 @@
 #include <algorithm>
 #include <atomic>
 #include <cstring>
+#include <initializer_list>
+#include <list>
 #include <map>
 #include <memory>
 #include <mutex>
@@ -27,6 +29,7 @@ using mmr::fail;
 namespace {
 
 constexpr size_t kTileAlign = 4096;
+constexpr size_t kMaxBindings = 64;  // unpinned device tables kept per context (least recently used go first)
 
 std::atomic<int64_t> g_next_store_id{0};  // NextStoreId, zuku_execute_context_impl.cc:86-89
 
@@ -36,29 +39,76 @@ struct TransposeRun {
   int64_t begin, count;
 };
 
+// A plan plus what does not depend on the buffers it will run on.
 struct DevicePlan {
   mmr_plan plan;
-  mmr_copy_chunk* d_copy16 = nullptr;
-  mmr_copy_chunk* d_generic = nullptr;
+  std::vector<uint32_t> copy_hints, span_hints;
+  std::vector<TransposeRun> transpose_runs;
+  mmr_copy_chunk* d_generic = nullptr;  // slot-relative tables, read through a launch's pointer table
   mmr_transpose_chunk* d_transposes = nullptr;
-  std::vector<TransposeRun> transpose_runs;  // the table is sorted by (itemsize, kind); one launch per run
-  bool tuned = false;                        // the table order has been chosen (timed or fixed by the options)
+  bool inline_copy = false, inline_span = false;  // the group table fits the kernel's argument block
+  uint64_t serial = 0;
+  uint64_t recent[8] = {};  // hashes of the buffer sets of the last launches that went without device tables
+  uint32_t recent_at = 0;
 
   DevicePlan() = default;
   DevicePlan(const DevicePlan&) = delete;
   DevicePlan& operator=(const DevicePlan&) = delete;
   ~DevicePlan() {  // hipFree waits for the device: launches that still read the tables finish first
-    (void)hipFree(d_copy16);
-    (void)hipFree(d_generic);
-    (void)hipFree(d_transposes);
+    if (d_generic) (void)hipFree(d_generic);
+    if (d_transposes) (void)hipFree(d_transposes);
+  }
+  bool needs_ptrs() const { return !plan.generic.empty() || !plan.transposes.empty(); }
+  // no launch of this plan can go without tables in device memory
+  bool needs_binding() const {
+    return needs_ptrs() || (plan.n_copy_chunks && !inline_copy) || (plan.n_span_chunks && !inline_span);
   }
 };
 
+// Where the tables of a launch lie inside one block of device memory (each 256-byte aligned).
+struct BlockLayout {
+  size_t ptrs = 0, cgroups = 0, cpieces = 0, chints = 0, sgroups = 0, smembers = 0, spieces = 0, shints = 0;
+  size_t generic = 0, transposes = 0;  // only with chunk tables included
+  size_t total = 0;
+};
+
+BlockLayout layout_block(const DevicePlan& dp, bool with_chunk_tables) {
+  const mmr_plan& p = dp.plan;
+  BlockLayout l;
+  size_t at = 0;
+  auto take = [&at](size_t bytes) {
+    const size_t here = at;
+    at += (bytes + 255) & ~static_cast<size_t>(255);
+    return here;
+  };
+  l.ptrs = take((dp.needs_ptrs() || with_chunk_tables) ? static_cast<size_t>(p.n_slots) * sizeof(void*) : 0);
+  l.cgroups = take(p.copy_groups.size() * sizeof(mmr::CopyGroup));
+  l.cpieces = take(p.copy_pieces.size() * sizeof(mmr::CopyPiece));
+  l.chints = take(dp.copy_hints.size() * sizeof(uint32_t));
+  l.sgroups = take(p.span_groups.size() * sizeof(mmr::SpanGroup));
+  l.smembers = take(p.span_members.size() * sizeof(mmr::SpanMember));
+  l.spieces = take(p.span_pieces.size() * sizeof(mmr::SpanPiece));
+  l.shints = take(dp.span_hints.size() * sizeof(uint32_t));
+  if (with_chunk_tables) {
+    l.generic = take(p.generic.size() * sizeof(mmr_copy_chunk));
+    l.transposes = take(p.transposes.size() * sizeof(mmr_transpose_chunk));
+  }
+  l.total = at;
+  return l;
+}
+
+// The device tables of a plan bound to one set of shard buffers: a pure function of (plan, buffer addresses), so
+// stores that come and go at the same addresses (buffers recycled through the cache) find their tables again.
 struct Binding {
   DevicePlan* plan = nullptr;
-  void** d_ptrs = nullptr;
-  std::vector<void*> host_ptrs;  // source of the upload; kept until the binding dies
-  std::vector<int64_t> store_ids;
+  std::vector<void*> ptrs;  // the key: every source and destination buffer, in slot order
+  char* d_block = nullptr;
+  size_t capacity = 0;
+  BlockLayout layout;
+  std::vector<char> host_block;  // source of the upload
+  hipEvent_t uploaded = nullptr;
+  bool pinned = false;  // made by mmr_reshard_bind or used under stream capture: never recycled
+  uint64_t last_use = 0;
 };
 
 struct CachedBuffer {
@@ -70,6 +120,7 @@ struct CachedBuffer {
 
 struct mmr_store {
   int64_t id = -1;
+  int64_t ordinal = -1;  // per context: the hash of the operation stream must not depend on other contexts
   std::string name;
   mmr_sharded_shape shape{};
   mmr::Side side;
@@ -90,23 +141,38 @@ struct mmr_context {
   hipStream_t stream = nullptr;
   bool owns_stream = false;
   hipEvent_t t0 = nullptr, t1 = nullptr;
+  std::vector<hipEvent_t> laps;  // mmr_timer_lap
+  size_t laps_used = 0;
   mmr_plan_options options{};
+  uint32_t flags = 0;
   std::mutex mu;
-  std::unordered_map<std::string, std::unique_ptr<DevicePlan>> plans;            // by descriptor pair(s)
-  std::map<std::vector<int64_t>, std::unique_ptr<Binding>> bindings;             // by store ids (src..., dst...)
-  std::unordered_map<std::string, std::vector<CachedBuffer>> buffer_cache;        // ArrayCache: by descriptor
+  std::unordered_map<std::string, std::unique_ptr<DevicePlan>> plans;  // by descriptor pair(s) and options
+  std::list<std::string> plan_lru;                                     // most recently used first
+  std::vector<std::unique_ptr<Binding>> bindings;
+  uint64_t clock = 0, next_plan_serial = 1;
+  std::unordered_map<std::string, std::vector<CachedBuffer>> buffer_cache;  // ArrayCache: by descriptor
+  std::unordered_map<std::string, std::vector<CachedBuffer>> host_cache;    // pinned buffers, by descriptor
+  // "use the cache as a store allocator" (ArrayCache::Make, zuku_execute_context_impl.cc:533-535): allocations of stores
+  // that were freed without keep_in_cache, by size; any new store of that size takes one (ordered on the stream behind
+  // the work of its previous owner), so a loop that creates and drops its output stores every step neither allocates
+  // nor frees.  mmr_clear_store_cache releases them.
+  std::unordered_map<size_t, std::vector<char*>> free_pool;
+  size_t free_pool_bytes = 0;
   std::unordered_map<int64_t, std::unique_ptr<mmr_store>> stores;
+  int64_t next_ordinal = 0;
   mmr_context_stats stats{};
   // mmr_reshard_batch_static: this GPU's static scratch array, a pinned staging buffer of the same size and the event
-  // that tells when the last copy out of the staging buffer is done; host-side plans (no device tables) by key
+  // that tells when the last copy out of the staging buffer is done
   char* static_scratch = nullptr;
   char* static_staging = nullptr;
   hipEvent_t static_copied = nullptr;
   bool static_copy_pending = false;
-  std::unordered_map<std::string, std::unique_ptr<mmr_plan>> static_plans;
 };
 
 namespace {
+
+constexpr size_t kMaxPlans = 256;  // cached plans per context (least recently used go first)
+constexpr size_t kFreePoolLimit = static_cast<size_t>(16) << 30;  // bytes the allocator keeps before it really frees
 
 #define MMR_HIP(expr)                                                                             \
   do {                                                                                            \
@@ -121,38 +187,68 @@ int use_device(mmr_context* ctx) {
   return MMR_OK;
 }
 
+bool capturing(mmr_context* ctx) {
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  return hipStreamIsCapturing(ctx->stream, &capture) == hipSuccess && capture != hipStreamCaptureStatusNone;
+}
+
+// Entry points that allocate, free, copy from pageable memory or wait may not run while the stream records a graph.
+int refuse_capture(mmr_context* ctx, const char* what) {
+  if (capturing(ctx))
+    return fail(MMR_INVALID_ARGUMENT, "%s is not allowed while the context's stream is capturing a graph", what);
+  return MMR_OK;
+}
+
 void account_alloc(mmr_context* ctx, int64_t bytes) {
   ctx->stats.bytes_allocated += bytes;
   ctx->stats.bytes_high_watermark = std::max(ctx->stats.bytes_high_watermark, ctx->stats.bytes_allocated);
+}
+
+int device_alloc(mmr_context* ctx, void** out, size_t bytes) {
+  MMR_HIP(hipMalloc(out, bytes));
+  ctx->stats.device_allocations += 1;
+  return MMR_OK;
+}
+
+// Makes the calling thread wait for the stream; counted, because the reference's calls are asynchronous.
+int blocking_sync(mmr_context* ctx) {
+  ctx->stats.host_blocking_syncs += 1;
+  MMR_HIP(hipStreamSynchronize(ctx->stream));
+  return MMR_OK;
+}
+
+void hash_op(mmr_context* ctx, uint64_t kind, std::initializer_list<uint64_t> values, const std::string* text = nullptr) {
+  if (!(ctx->flags & MMR_CHECK_INVARIANTS)) return;
+  uint64_t h = static_cast<uint64_t>(ctx->stats.operation_hash);
+  auto mix = [&h](uint64_t v) {  // FNV-1a over the 8 bytes of v
+    for (int i = 0; i < 8; ++i) {
+      h ^= (v >> (8 * i)) & 0xff;
+      h *= 0x100000001b3ull;
+    }
+  };
+  if (h == 0) h = 0xcbf29ce484222325ull;
+  mix(kind);
+  for (uint64_t v : values) mix(v);
+  if (text)
+    for (unsigned char c : *text) mix(c);
+  ctx->stats.operation_hash = static_cast<int64_t>(h);
 }
 
 template <class T>
 int upload(mmr_context* ctx, const std::vector<T>& host, T** dev) {
   *dev = nullptr;
   if (host.empty()) return MMR_OK;
-  MMR_HIP(hipMalloc(reinterpret_cast<void**>(dev), host.size() * sizeof(T)));
+  if (int rc = device_alloc(ctx, reinterpret_cast<void**>(dev), host.size() * sizeof(T))) return rc;
   MMR_HIP(hipMemcpyAsync(*dev, host.data(), host.size() * sizeof(T), hipMemcpyHostToDevice, ctx->stream));
   // callers pass vectors that live as long as the device copy does
   return MMR_OK;
 }
 
-void drop_bindings_of(mmr_context* ctx, int64_t store_id) {
-  for (auto it = ctx->bindings.begin(); it != ctx->bindings.end();) {
-    const auto& ids = it->second->store_ids;
-    if (std::find(ids.begin(), ids.end(), store_id) != ids.end()) {
-      (void)hipFree(it->second->d_ptrs);  // hipFree waits for the device, in-flight launches finish first
-      it = ctx->bindings.erase(it);
-    } else {
-      ++it;
-    }
-  }
-}
-
-// The transpose kernel's LDS tile and lane mapping assume bounds the planner keeps; checked before every first
-// launch of a plan.  Also splits the table into runs of equal element width and kind, one launch each.
+// The transpose kernel's LDS tile and lane mapping assume bounds the planner keeps; checked before the first launch
+// of a plan.  Also splits the table into runs of equal element width and kind, one launch each.
 int check_transposes(const mmr_plan& plan, std::vector<TransposeRun>* runs) {
   const std::vector<mmr_transpose_chunk>& tr = plan.transposes;
-  for (const mmr_transpose_chunk& c : tr) {  // the kernel's LDS tile and lane mapping assume these bounds
+  for (const mmr_transpose_chunk& c : tr) {
     uint32_t tile_x = 0, tile_y = 0;
     mmr::transpose_tile_extent(c.itemsize, &tile_x, &tile_y);
     const bool width_ok = c.itemsize == 1 || c.itemsize == 2 || c.itemsize == 4 || c.itemsize == 8 || c.itemsize == 16;
@@ -176,128 +272,312 @@ int check_transposes(const mmr_plan& plan, std::vector<TransposeRun>* runs) {
   return MMR_OK;
 }
 
-// Plans n descriptor pairs under `options` and uploads the tables (not cached here).
-int make_device_plan(mmr_context* ctx, const std::vector<mmr_sharded_shape>& srcs, const std::vector<mmr_sharded_shape>& dsts,
-                     const mmr_plan_options& options, DevicePlan* dp) {
-  const int n = static_cast<int>(srcs.size());
-  if (int rc = mmr::build_plan(srcs.data(), dsts.data(), n, options, &dp->plan)) return rc;
-  if (int rc = check_transposes(dp->plan, &dp->transpose_runs)) return rc;
-  if (int rc = upload(ctx, dp->plan.copy16, &dp->d_copy16)) return rc;
-  if (int rc = upload(ctx, dp->plan.generic, &dp->d_generic)) return rc;
-  if (int rc = upload(ctx, dp->plan.transposes, &dp->d_transposes)) return rc;
+// What the span kernel's LDS staging assumes.
+int check_spans(const mmr_plan& plan) {
+  for (const mmr::SpanGroup& g : plan.span_groups)
+    if (g.span == 0 || g.span > mmr::kSpanMaxBytes || g.head == 0 || g.head > g.span || g.W == 0 ||
+        g.W > mmr::kSpanMaxRowBytes)
+      return fail(MMR_INTERNAL, "span group with span %u, head %u, row %u", g.span, g.head, g.W);
   return MMR_OK;
 }
 
+// Plans n descriptor pairs under `options`; the chunk tables that need no binding are uploaded.  With
+// `device_tables` false nothing touches the device (the static entry point brings its own memory).
+int make_device_plan(mmr_context* ctx, const std::vector<mmr_sharded_shape>& srcs, const std::vector<mmr_sharded_shape>& dsts,
+                     const mmr_plan_options& options, bool device_tables, DevicePlan* dp) {
+  const int n = static_cast<int>(srcs.size());
+  if (int rc = mmr::build_plan(srcs.data(), dsts.data(), n, options, &dp->plan)) return rc;
+  if (int rc = check_transposes(dp->plan, &dp->transpose_runs)) return rc;
+  if (int rc = check_spans(dp->plan)) return rc;
+  const mmr_plan& p = dp->plan;
+  const bool may_inline = !(options.flags & MMR_PLAN_NO_INLINE);  // without it every launch builds device tables
+  dp->inline_copy = may_inline && p.copy_groups.size() <= mmr::kInlineCopyGroups && p.copy_pieces.size() <= mmr::kInlineCopyPieces;
+  dp->inline_span = may_inline && p.span_groups.size() <= mmr::kInlineSpanGroups &&
+                    p.span_members.size() <= mmr::kInlineSpanMembers && p.span_pieces.size() <= mmr::kInlineSpanPieces;
+  dp->copy_hints = mmr::group_hints(p.copy_groups, p.n_copy_chunks);
+  dp->span_hints = mmr::group_hints(p.span_groups, p.n_span_chunks);
+  dp->serial = ctx->next_plan_serial++;
+  if (device_tables) {
+    if (int rc = upload(ctx, dp->plan.generic, &dp->d_generic)) return rc;
+    if (int rc = upload(ctx, dp->plan.transposes, &dp->d_transposes)) return rc;
+  }
+  return MMR_OK;
+}
+
+void drop_bindings_of_plan(mmr_context* ctx, const DevicePlan* dp);
+
 int get_plan(mmr_context* ctx, const std::vector<mmr_sharded_shape>& srcs, const std::vector<mmr_sharded_shape>& dsts,
-             DevicePlan** out) {
+             DevicePlan** out, std::string* key_out = nullptr) {
   const int n = static_cast<int>(srcs.size());
   std::string key = mmr::plan_key(srcs.data(), dsts.data(), n, ctx->options);
+  if (key_out) *key_out = key;
   auto it = ctx->plans.find(key);
   if (it != ctx->plans.end()) {
     ctx->stats.plan_cache_hits += 1;
     *out = it->second.get();
+    auto pos = std::find(ctx->plan_lru.begin(), ctx->plan_lru.end(), key);
+    if (pos != ctx->plan_lru.begin() && pos != ctx->plan_lru.end()) ctx->plan_lru.splice(ctx->plan_lru.begin(), ctx->plan_lru, pos);
     return MMR_OK;
   }
+  if (capturing(ctx))  // building a plan may allocate and copy
+    return fail(MMR_INVALID_ARGUMENT,
+                "the stream is capturing and this reshard has no cached plan yet: call mmr_reshard_bind (or run the "
+                "reshard once) before the capture begins");
   auto dp = std::make_unique<DevicePlan>();
-  if (int rc = make_device_plan(ctx, srcs, dsts, ctx->options, dp.get())) return rc;
+  if (int rc = make_device_plan(ctx, srcs, dsts, ctx->options, true, dp.get())) return rc;
   ctx->stats.plans_built += 1;
   *out = dp.get();
-  ctx->plans.emplace(std::move(key), std::move(dp));
+  ctx->plans.emplace(key, std::move(dp));
+  ctx->plan_lru.push_front(std::move(key));
+  // Least recently used plans go when the cache is full.  Only plans without device state of their own and without
+  // bindings can go without waiting for the device; the others stay until mmr_context_clear_plans.
+  if (ctx->plans.size() > kMaxPlans) {
+    for (auto pos = std::prev(ctx->plan_lru.end()); pos != ctx->plan_lru.begin();) {
+      auto victim = ctx->plans.find(*pos);
+      auto prev = std::prev(pos);
+      bool bound = false;
+      for (const auto& b : ctx->bindings) bound |= b->plan == victim->second.get();
+      if (!bound && !victim->second->d_generic && !victim->second->d_transposes) {
+        ctx->plans.erase(victim);
+        ctx->plan_lru.erase(pos);
+        if (ctx->plans.size() <= kMaxPlans) break;
+      }
+      pos = prev;
+    }
+  }
+  ctx->stats.plans_cached = static_cast<int64_t>(ctx->plans.size());
   return MMR_OK;
 }
 
-// One launch per kernel class over the tables of plan `p` as they lie in device memory.
-int launch_tables(mmr_context* ctx, const mmr_plan& p, const mmr_copy_chunk* d_copy16, const mmr_copy_chunk* d_generic,
-                  const mmr_transpose_chunk* d_transposes, const std::vector<TransposeRun>& runs, void* const* d_ptrs) {
-  const uint32_t xm = p.options.xcd_mode;
-  // aligned chunks: runs of 64 table neighbours per XCD measured best across the benchmark configurations
-  MMR_HIP(mmr::launch_copy16(d_copy16, static_cast<int64_t>(p.copy16.size()), d_ptrs, xm == 0 ? 64 : xm, ctx->stream));
-  // generic chunks leave partial lines at run boundaries and share source lines with the chunks of neighbouring
-  // destination tiles; table neighbours merge both when they share an L2: runs of 64 per XCD (measured)
-  MMR_HIP(mmr::launch_copy_generic(d_generic, static_cast<int64_t>(p.generic.size()), d_ptrs, xm == 0 ? 64 : xm, ctx->stream));
-  for (const TransposeRun& run : runs)
+// Slot -> buffer address for the stores of a batch.
+void collect_ptrs(const mmr_plan& p, mmr_store* const* srcs, mmr_store* const* dsts, int n, std::vector<void*>* ptrs) {
+  ptrs->assign(static_cast<size_t>(p.n_slots), nullptr);
+  for (int a = 0; a < n; ++a) {
+    size_t slot = static_cast<size_t>(p.slot_bases[a]);
+    for (int64_t k = 0; k < srcs[a]->side.dev_count; ++k) (*ptrs)[slot++] = srcs[a]->tile(k);
+    for (int64_t k = 0; k < dsts[a]->side.dev_count; ++k) (*ptrs)[slot++] = dsts[a]->tile(k);
+  }
+}
+
+uint64_t address_of(const std::vector<void*>& ptrs, uint32_t slot, uint64_t off) {
+  return slot == MMR_SLOT_FILL ? 0 : reinterpret_cast<uint64_t>(ptrs[slot]) + off;
+}
+
+void bind_copy_pieces(const mmr::CopyPiece* in, size_t n, const std::vector<void*>& ptrs, mmr::CopyPiece* out) {
+  for (size_t i = 0; i < n; ++i) {
+    out[i] = in[i];
+    out[i].src = address_of(ptrs, in[i].src_slot, in[i].src);
+    out[i].dst = address_of(ptrs, in[i].dst_slot, in[i].dst);
+  }
+}
+
+void bind_span_tables(const mmr_plan& p, const std::vector<void*>& ptrs, mmr::SpanMember* members, mmr::SpanPiece* pieces) {
+  for (size_t i = 0; i < p.span_members.size(); ++i) {
+    members[i] = p.span_members[i];
+    members[i].dst = address_of(ptrs, p.span_members[i].dst_slot, p.span_members[i].dst);
+  }
+  for (size_t i = 0; i < p.span_pieces.size(); ++i) {
+    pieces[i] = p.span_pieces[i];
+    pieces[i].src = address_of(ptrs, p.span_pieces[i].src_slot, p.span_pieces[i].src);
+  }
+}
+
+// Fills `block` (layout l) with the tables of dp bound to ptrs.
+void fill_block(const DevicePlan& dp, const BlockLayout& l, const std::vector<void*>& ptrs, bool with_chunk_tables, char* block) {
+  const mmr_plan& p = dp.plan;
+  if (dp.needs_ptrs() || with_chunk_tables) std::memcpy(block + l.ptrs, ptrs.data(), ptrs.size() * sizeof(void*));
+  if (!p.copy_groups.empty()) {
+    std::memcpy(block + l.cgroups, p.copy_groups.data(), p.copy_groups.size() * sizeof(mmr::CopyGroup));
+    bind_copy_pieces(p.copy_pieces.data(), p.copy_pieces.size(), ptrs, reinterpret_cast<mmr::CopyPiece*>(block + l.cpieces));
+    std::memcpy(block + l.chints, dp.copy_hints.data(), dp.copy_hints.size() * sizeof(uint32_t));
+  }
+  if (!p.span_groups.empty()) {
+    std::memcpy(block + l.sgroups, p.span_groups.data(), p.span_groups.size() * sizeof(mmr::SpanGroup));
+    bind_span_tables(p, ptrs, reinterpret_cast<mmr::SpanMember*>(block + l.smembers),
+                     reinterpret_cast<mmr::SpanPiece*>(block + l.spieces));
+    std::memcpy(block + l.shints, dp.span_hints.data(), dp.span_hints.size() * sizeof(uint32_t));
+  }
+  if (with_chunk_tables) {
+    if (!p.generic.empty()) std::memcpy(block + l.generic, p.generic.data(), p.generic.size() * sizeof(mmr_copy_chunk));
+    if (!p.transposes.empty())
+      std::memcpy(block + l.transposes, p.transposes.data(), p.transposes.size() * sizeof(mmr_transpose_chunk));
+  }
+}
+
+void drop_bindings_of_plan(mmr_context* ctx, const DevicePlan* dp) {
+  for (auto it = ctx->bindings.begin(); it != ctx->bindings.end();) {
+    if ((*it)->plan == dp) {
+      (void)hipFree((*it)->d_block);  // waits for the device: launches that still read the tables finish first
+      if ((*it)->uploaded) (void)hipEventDestroy((*it)->uploaded);
+      it = ctx->bindings.erase(it);
+    } else {
+      ++it;
+    }
+  }
+  ctx->stats.bindings_cached = static_cast<int64_t>(ctx->bindings.size());
+}
+
+// The binding of dp to ptrs: cached, else built in a recycled or new block and uploaded on the stream.
+int get_binding(mmr_context* ctx, DevicePlan* dp, const std::vector<void*>& ptrs, bool pin, bool count_hit, Binding** out) {
+  for (auto& b : ctx->bindings)
+    if (b->plan == dp && b->ptrs == ptrs) {
+      b->last_use = ++ctx->clock;
+      b->pinned |= pin || capturing(ctx);
+      if (count_hit) ctx->stats.binding_cache_hits += 1;
+      *out = b.get();
+      return MMR_OK;
+    }
+  if (capturing(ctx))
+    return fail(MMR_INVALID_ARGUMENT,
+                "the stream is capturing and this reshard has no bound device tables yet: call mmr_reshard_bind (or "
+                "run the reshard once) before the capture begins");
+  const BlockLayout l = layout_block(*dp, false);
+  // a block to put it in: the least recently used unpinned binding's once the cache is full, else a new one
+  std::unique_ptr<Binding> b;
+  size_t unpinned = 0;
+  for (auto& x : ctx->bindings) unpinned += x->pinned ? 0 : 1;
+  if (unpinned >= kMaxBindings) {
+    size_t victim = ctx->bindings.size();
+    for (size_t i = 0; i < ctx->bindings.size(); ++i)
+      if (!ctx->bindings[i]->pinned && (victim == ctx->bindings.size() || ctx->bindings[i]->last_use < ctx->bindings[victim]->last_use))
+        victim = i;
+    b = std::move(ctx->bindings[victim]);
+    ctx->bindings.erase(ctx->bindings.begin() + static_cast<std::ptrdiff_t>(victim));
+    // its last upload read host_block: long done, but make sure before the vector is rewritten
+    if (hipEventQuery(b->uploaded) != hipSuccess) {
+      ctx->stats.host_blocking_syncs += 1;
+      MMR_HIP(hipEventSynchronize(b->uploaded));
+    }
+    if (b->capacity < l.total) {  // too small: this one does cost a device-wide wait
+      MMR_HIP(hipFree(b->d_block));
+      b->d_block = nullptr;
+      b->capacity = 0;
+    }
+  } else {
+    b = std::make_unique<Binding>();
+    MMR_HIP(hipEventCreateWithFlags(&b->uploaded, hipEventDisableTiming));
+  }
+  if (!b->d_block) {
+    const size_t capacity = std::max<size_t>(l.total, 16384);
+    if (int rc = device_alloc(ctx, reinterpret_cast<void**>(&b->d_block), capacity)) {
+      (void)hipEventDestroy(b->uploaded);
+      return rc;
+    }
+    b->capacity = capacity;
+  }
+  b->plan = dp;
+  b->ptrs = ptrs;
+  b->layout = l;
+  b->pinned = pin;
+  b->last_use = ++ctx->clock;
+  b->host_block.assign(l.total, 0);
+  fill_block(*dp, l, ptrs, false, b->host_block.data());
+  // stream-ordered: launches queued earlier that still read a recycled block finish before the copy overwrites it
+  hipError_t e = hipMemcpyAsync(b->d_block, b->host_block.data(), l.total, hipMemcpyHostToDevice, ctx->stream);
+  if (e == hipSuccess) e = hipEventRecord(b->uploaded, ctx->stream);
+  if (e != hipSuccess) {
+    (void)hipFree(b->d_block);
+    (void)hipEventDestroy(b->uploaded);
+    return fail(MMR_HIP_ERROR, "upload of the bound tables failed: %s", hipGetErrorString(e));
+  }
+  ctx->stats.bindings_built += 1;
+  *out = b.get();
+  ctx->bindings.push_back(std::move(b));
+  ctx->stats.bindings_cached = static_cast<int64_t>(ctx->bindings.size());
+  return MMR_OK;
+}
+
+// Launches over tables in device memory: `block` laid out by l; the generic and transpose chunk tables at the
+// given addresses.
+int launch_block(mmr_context* ctx, const DevicePlan& dp, const char* block, const BlockLayout& l,
+                 const mmr_copy_chunk* d_generic, const mmr_transpose_chunk* d_transposes, bool copies, bool spans) {
+  const mmr_plan& p = dp.plan;
+  const uint32_t xm = p.options.xcd_mode == 0 ? 64 : p.options.xcd_mode;  // runs of 64 table neighbours per XCD (measured)
+  if (copies && p.n_copy_chunks) {
+    uint32_t starts[mmr::kMaxDirectGroups];
+    const bool direct = p.copy_groups.size() <= mmr::kMaxDirectGroups;
+    for (size_t i = 0; direct && i < p.copy_groups.size(); ++i) starts[i] = p.copy_groups[i].first_chunk;
+    MMR_HIP(mmr::launch_copy_groups(reinterpret_cast<const mmr::CopyGroup*>(block + l.cgroups),
+                                    static_cast<uint32_t>(p.copy_groups.size()),
+                                    reinterpret_cast<const mmr::CopyPiece*>(block + l.cpieces),
+                                    reinterpret_cast<const uint32_t*>(block + l.chints), direct ? starts : nullptr,
+                                    p.n_copy_chunks, xm, ctx->stream));
+  }
+  if (spans && p.n_span_chunks)
+    MMR_HIP(mmr::launch_spans(reinterpret_cast<const mmr::SpanGroup*>(block + l.sgroups),
+                              static_cast<uint32_t>(p.span_groups.size()),
+                              reinterpret_cast<const mmr::SpanMember*>(block + l.smembers),
+                              reinterpret_cast<const mmr::SpanPiece*>(block + l.spieces),
+                              reinterpret_cast<const uint32_t*>(block + l.shints), p.n_span_chunks, xm, ctx->stream));
+  void* const* d_ptrs = reinterpret_cast<void* const*>(block + l.ptrs);
+  MMR_HIP(mmr::launch_copy_generic(d_generic, static_cast<int64_t>(p.generic.size()), d_ptrs, xm, ctx->stream));
+  for (const TransposeRun& run : dp.transpose_runs)
     // tiles are ordered in 8 x 8 blocks; runs of 64 table neighbours per XCD keep a block in one L2 (measured best)
-    MMR_HIP(mmr::launch_transpose(d_transposes + run.begin, run.count, d_ptrs, xm == 0 ? 64 : xm, run.itemsize,
-                                  run.vector_only, ctx->stream));
+    MMR_HIP(mmr::launch_transpose(d_transposes + run.begin, run.count, d_ptrs, xm, run.itemsize, run.vector_only, ctx->stream));
   return MMR_OK;
-}
-
-int launch_plan(mmr_context* ctx, const DevicePlan* dp, void* const* d_ptrs) {
-  return launch_tables(ctx, dp->plan, dp->d_copy16, dp->d_generic, dp->d_transposes, dp->transpose_runs, d_ptrs);
 }
 
 int64_t launches_of(const DevicePlan* dp) {
-  return (dp->plan.copy16.empty() ? 0 : 1) + (dp->plan.generic.empty() ? 0 : 1) +
+  return (dp->plan.n_copy_chunks ? 1 : 0) + (dp->plan.n_span_chunks ? 1 : 0) + (dp->plan.generic.empty() ? 0 : 1) +
          static_cast<int64_t>(dp->transpose_runs.size());
 }
 
-// Which order of the chunk tables is fastest depends on how the two tilings interleave in memory (measured: plain
-// destination order for configurations 1, 2 and 4, destination tiles interleaved in 4 MiB fractions for
-// configuration 3, in 64 KiB fractions for ragged rows).  The first reshard of a descriptor pair therefore times a
-// few orders on the caller's own buffers (a reshard is idempotent) and keeps the fastest; the choice is cached with
-// the plan.  Blocks the calling thread for those few launches.
-int tune_plan(mmr_context* ctx, DevicePlan* dp, void* const* d_ptrs) {
-  dp->tuned = true;
-  const mmr_plan_options base = dp->plan.options;
-  const size_t chunks = dp->plan.copy16.size() + dp->plan.generic.size();
-  if (base.order != 0 || (base.flags & MMR_PLAN_NO_AUTOTUNE) || chunks < 1024 || chunks > 262144) return MMR_OK;
-  struct Candidate {
-    uint32_t order, kib;
-  };
-  const Candidate candidates[] = {{4, 64}, {4, 1024}, {4, 4096}, {2, 0}};
-  hipEvent_t e0 = nullptr, e1 = nullptr;
-  MMR_HIP(hipEventCreate(&e0));
-  MMR_HIP(hipEventCreate(&e1));
-  int reps = 3;  // launches per measurement; raised after the first one so that a measurement spans ~0.5 ms
-  auto time_plan = [&](const DevicePlan* plan, float* ms) -> int {
-    if (int rc = launch_plan(ctx, plan, d_ptrs)) return rc;  // warm-up
-    MMR_HIP(hipEventRecord(e0, ctx->stream));
-    for (int i = 0; i < reps; ++i)
-      if (int rc = launch_plan(ctx, plan, d_ptrs)) return rc;
-    MMR_HIP(hipEventRecord(e1, ctx->stream));
-    MMR_HIP(hipEventSynchronize(e1));
-    MMR_HIP(hipEventElapsedTime(ms, e0, e1));
-    *ms /= static_cast<float>(reps);
-    return MMR_OK;
-  };
-  int rc = MMR_OK;
-  float best_ms = 0;
-  int64_t timed = 1;
-  rc = time_plan(dp, &best_ms);
-  if (rc == MMR_OK && best_ms > 0 && best_ms * 3 < 0.5f) {  // short kernels: average over more launches
-    reps = std::min(24, static_cast<int>(0.5f / best_ms) + 1);
-    rc = time_plan(dp, &best_ms);
-  }
-  std::unique_ptr<DevicePlan> best;
-  for (const Candidate& cand : candidates) {
-    if (rc != MMR_OK) break;
-    if (cand.order == 2 && dp->plan.generic.empty()) continue;  // the default already is order 2 for aligned chunks
-    if (cand.order == 4 && cand.kib == 64 && dp->plan.copy16.empty()) continue;  // ... and 4 / 64 KiB for ragged ones
-    mmr_plan_options o = base;
-    o.order = cand.order;
-    o.flags = (o.flags & 0xffu) | (cand.kib << 8);
-    auto alt = std::make_unique<DevicePlan>();
-    rc = make_device_plan(ctx, dp->plan.srcs, dp->plan.dsts, o, alt.get());
-    float ms = 0;
-    if (rc == MMR_OK) rc = time_plan(alt.get(), &ms);
-    if (rc == MMR_OK) timed += 1;
-    if (rc == MMR_OK && ms < 0.98f * best_ms) {  // only a clear win replaces the default
-      best_ms = ms;
-      best = std::move(alt);
+Binding* find_binding(mmr_context* ctx, const DevicePlan* dp, const std::vector<void*>& ptrs) {
+  for (auto& b : ctx->bindings)
+    if (b->plan == dp && b->ptrs == ptrs) return b.get();
+  return nullptr;
+}
+
+// One launch per kernel class.  Tables in device memory, bound to these buffers, are the fast way (a workgroup's
+// table reads stay in the caches); they cost an allocation and an upload the first time.  Group tables small enough
+// can instead travel in the kernel's argument block, bound right here: nothing to allocate, upload or keep alive
+// (about a microsecond slower per launch).  So: the first launch of a plan on a set of buffers goes through the
+// argument block where it can, the second one on the same buffers builds the device tables, and every later one
+// finds them (as does any launch after mmr_reshard_bind).  `tables`: 0 = that policy, 1 = device tables now.
+int launch_plan(mmr_context* ctx, DevicePlan* dp, const std::vector<void*>& ptrs, int tables, bool count_hit) {
+  const mmr_plan& p = dp->plan;
+  const uint32_t xm = p.options.xcd_mode == 0 ? 64 : p.options.xcd_mode;
+  Binding* binding = find_binding(ctx, dp, ptrs);
+  if (binding) {
+    binding->last_use = ++ctx->clock;
+    binding->pinned |= capturing(ctx);
+    if (count_hit) ctx->stats.binding_cache_hits += 1;
+  } else {
+    bool want = dp->needs_binding() || tables == 1;
+    if (!want && !capturing(ctx)) {  // seen these buffers before?
+      uint64_t h = 0xcbf29ce484222325ull;
+      for (void* q : ptrs) h = (h ^ reinterpret_cast<uint64_t>(q)) * 0x100000001b3ull;
+      h |= 1;
+      for (uint64_t r : dp->recent) want |= r == h;
+      if (!want) dp->recent[dp->recent_at++ % 8] = h;
     }
+    if (want)
+      if (int rc = get_binding(ctx, dp, ptrs, /*pin=*/false, /*count_hit=*/false, &binding)) return rc;
   }
-  (void)hipEventDestroy(e0);
-  (void)hipEventDestroy(e1);
-  if (rc == MMR_OK && best) {  // the cached object keeps its address (bindings point at it) and takes the winner's tables
-    std::swap(dp->plan, best->plan);
-    std::swap(dp->d_copy16, best->d_copy16);
-    std::swap(dp->d_generic, best->d_generic);
-    std::swap(dp->d_transposes, best->d_transposes);
-    std::swap(dp->transpose_runs, best->transpose_runs);
-    dp->plan.options = base;  // still the plan of the context's options
+  const bool inline_copy = !binding && dp->inline_copy, inline_span = !binding && dp->inline_span;
+  if (p.n_copy_chunks && inline_copy) {
+    mmr::InlineCopyTable t{};
+    t.n_groups = static_cast<uint32_t>(p.copy_groups.size());
+    t.n_chunks = p.n_copy_chunks;
+    std::copy(p.copy_groups.begin(), p.copy_groups.end(), t.groups);
+    bind_copy_pieces(p.copy_pieces.data(), p.copy_pieces.size(), ptrs, t.pieces);
+    MMR_HIP(mmr::launch_copy_groups_inline(t, xm, ctx->stream));
+    ctx->stats.inline_launches += 1;
   }
-  dp->plan.stats.orders_timed = timed;
-  return rc;
+  if (p.n_span_chunks && inline_span) {
+    mmr::InlineSpanTable t{};
+    t.n_groups = static_cast<uint32_t>(p.span_groups.size());
+    t.n_chunks = p.n_span_chunks;
+    std::copy(p.span_groups.begin(), p.span_groups.end(), t.groups);
+    bind_span_tables(p, ptrs, t.members, t.pieces);
+    MMR_HIP(mmr::launch_spans_inline(t, xm, ctx->stream));
+    ctx->stats.inline_launches += 1;
+  }
+  if (binding)
+    if (int rc = launch_block(ctx, *dp, binding->d_block, binding->layout, dp->d_generic, dp->d_transposes, true, true))
+      return rc;
+  ctx->stats.kernel_launches += launches_of(dp);
+  return MMR_OK;
 }
 
 int check_store(mmr_context* ctx, const mmr_store* s, const char* what) {
@@ -322,130 +602,184 @@ int check_batch(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts
       if (dsts[a] == srcs[b] || (a != b && dsts[a] == dsts[b]))
         return fail(MMR_INVALID_ARGUMENT, "store %lld is written by array %d and used again by array %d of the same batch",
                     (long long)dsts[a]->id, a, b);
+  if (ctx->flags & MMR_CHECK_INVARIANTS) {
+    // mm_mock_mm_xla.cc:347-369: every operand holds a tile on each device of its list
+    for (int a = 0; a < n; ++a)
+      for (mmr_store* s : {srcs[a], dsts[a]}) {
+        ctx->stats.invariant_checks += 1;
+        for (int64_t k = 0; k < s->side.dev_count; ++k)
+          if (s->side.shard_bytes > 0 && !s->tile(k))
+            return fail(MMR_INTERNAL, "invariant violated: store %lld has no tile on device %lld", (long long)s->id,
+                        (long long)(s->side.dev_start + k));
+        hash_op(ctx, 2 /* Reshard */, {static_cast<uint64_t>(s->ordinal)}, &s->shape_key);
+      }
+  }
   return MMR_OK;
+}
+
+void shapes_of(mmr_store* const* srcs, mmr_store* const* dsts, int n, std::vector<mmr_sharded_shape>* s,
+               std::vector<mmr_sharded_shape>* d) {
+  s->resize(static_cast<size_t>(n));
+  d->resize(static_cast<size_t>(n));
+  for (int a = 0; a < n; ++a) {
+    (*s)[a] = srcs[a]->shape;
+    (*d)[a] = dsts[a]->shape;
+  }
 }
 
 int reshard_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int n, bool launch = true) {
   if (n == 0) return MMR_OK;
   if (int rc = use_device(ctx)) return rc;
   if (int rc = check_batch(ctx, srcs, dsts, n)) return rc;
-  std::vector<int64_t> ids;
-  ids.reserve(2 * n);
-  for (int a = 0; a < n; ++a) ids.push_back(srcs[a]->id);
-  for (int a = 0; a < n; ++a) ids.push_back(dsts[a]->id);
+  std::vector<mmr_sharded_shape> sshapes, dshapes;
+  shapes_of(srcs, dsts, n, &sshapes, &dshapes);
+  DevicePlan* dp = nullptr;
+  if (int rc = get_plan(ctx, sshapes, dshapes, &dp)) return rc;
+  std::vector<void*> ptrs;
+  collect_ptrs(dp->plan, srcs, dsts, n, &ptrs);
+  if (!launch) {  // mmr_reshard_bind: everything but the launches; the tables stay until the plans are cleared
+    Binding* binding = nullptr;
+    return get_binding(ctx, dp, ptrs, /*pin=*/true, /*count_hit=*/false, &binding);
+  }
+  ctx->stats.reshard_calls += 1;
+  return launch_plan(ctx, dp, ptrs, /*tables=*/0, /*count_hit=*/true);
+}
 
-  if (launch) ctx->stats.reshard_calls += 1;
-  Binding* binding = nullptr;
-  auto bit = ctx->bindings.find(ids);
-  if (bit != ctx->bindings.end()) {
-    binding = bit->second.get();
-    if (launch) ctx->stats.binding_cache_hits += 1;
-  } else {
-    // Building a plan or a pointer table allocates and copies: not allowed while the stream records a graph.
-    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(ctx->stream, &capture) == hipSuccess && capture != hipStreamCaptureStatusNone)
-      return fail(MMR_INVALID_ARGUMENT,
-                  "the stream is capturing and this reshard has no cached plan and pointer table yet: "
-                  "call mmr_reshard_bind (or run the reshard once) before the capture begins");
-    std::vector<mmr_sharded_shape> sshapes(n), dshapes(n);
-    for (int a = 0; a < n; ++a) {
-      sshapes[a] = srcs[a]->shape;
-      dshapes[a] = dsts[a]->shape;
-    }
-    DevicePlan* dp = nullptr;
-    if (int rc = get_plan(ctx, sshapes, dshapes, &dp)) return rc;
-    std::vector<void*> ptrs(static_cast<size_t>(dp->plan.n_slots));
-    for (int a = 0; a < n; ++a) {
-      size_t slot = static_cast<size_t>(dp->plan.slot_bases[a]);
-      for (int64_t k = 0; k < srcs[a]->side.dev_count; ++k) ptrs[slot++] = srcs[a]->tile(k);
-      for (int64_t k = 0; k < dsts[a]->side.dev_count; ++k) ptrs[slot++] = dsts[a]->tile(k);
-    }
-    auto b = std::make_unique<Binding>();
-    b->plan = dp;
-    b->store_ids = ids;
-    b->host_ptrs = std::move(ptrs);
-    if (int rc = upload(ctx, b->host_ptrs, &b->d_ptrs)) return rc;
-    ctx->stats.bindings_built += 1;
-    binding = b.get();
-    ctx->bindings.emplace(ids, std::move(b));
+// mmr_reshard_tune: times the default order and a few interleaved ones on the caller's buffers.
+int tune_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int n, int64_t* order_used) {
+  if (int rc = use_device(ctx)) return rc;
+  if (int rc = refuse_capture(ctx, "mmr_reshard_tune")) return rc;
+  if (int rc = check_batch(ctx, srcs, dsts, n)) return rc;
+  std::vector<mmr_sharded_shape> sshapes, dshapes;
+  shapes_of(srcs, dsts, n, &sshapes, &dshapes);
+  DevicePlan* dp = nullptr;
+  std::string key;
+  if (int rc = get_plan(ctx, sshapes, dshapes, &dp, &key)) return rc;
+  const mmr_plan_options base = dp->plan.options;
+  if (order_used) *order_used = dp->plan.stats.order_used;
+  const size_t chunks = static_cast<size_t>(dp->plan.n_copy_chunks) + dp->plan.n_span_chunks + dp->plan.generic.size();
+  if (base.order != 0 || chunks < 1024) return MMR_OK;  // a fixed order, or too small to matter
+  std::vector<void*> ptrs;
+  collect_ptrs(dp->plan, srcs, dsts, n, &ptrs);
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  MMR_HIP(hipEventCreate(&e0));
+  if (hipEventCreate(&e1) != hipSuccess) {
+    (void)hipEventDestroy(e0);
+    return fail(MMR_HIP_ERROR, "hipEventCreate failed");
   }
-  if (!launch) return MMR_OK;
-  DevicePlan* dp = binding->plan;
-  if (!dp->tuned) {
-    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(ctx->stream, &capture) == hipSuccess && capture != hipStreamCaptureStatusNone) {
-      // recorded into a graph as it is: the graph keeps the addresses of these tables, so they must never be
-      // replaced by a later tuning run
-      dp->tuned = true;
-    } else if (int rc = tune_plan(ctx, dp, binding->d_ptrs)) {
-      return rc;
-    }
+  int reps = 3;  // launches per measurement; raised after the first one so that a measurement spans ~0.5 ms
+  auto time_plan = [&](DevicePlan* plan, float* ms) -> int {
+    if (int rc = launch_plan(ctx, plan, ptrs, 1, false)) return rc;  // warm-up (and upload of its tables)
+    MMR_HIP(hipEventRecord(e0, ctx->stream));
+    for (int i = 0; i < reps; ++i)
+      if (int rc = launch_plan(ctx, plan, ptrs, 1, false)) return rc;
+    MMR_HIP(hipEventRecord(e1, ctx->stream));
+    ctx->stats.host_blocking_syncs += 1;
+    MMR_HIP(hipEventSynchronize(e1));
+    MMR_HIP(hipEventElapsedTime(ms, e0, e1));
+    *ms /= static_cast<float>(reps);
+    return MMR_OK;
+  };
+  float best_ms = 0;
+  int64_t timed = 0;
+  int rc = time_plan(dp, &best_ms);
+  if (rc == MMR_OK && best_ms > 0 && best_ms * 3 < 0.5f) {  // short kernels: average over more launches
+    reps = std::min(24, static_cast<int>(0.5f / best_ms) + 1);
+    rc = time_plan(dp, &best_ms);
   }
-  if (int rc = launch_plan(ctx, dp, binding->d_ptrs)) return rc;
-  ctx->stats.kernel_launches += launches_of(dp);
+  if (rc != MMR_OK) {  // the default plan itself does not run: report it
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return rc;
+  }
+  timed = 1;
+  struct Candidate {
+    uint32_t order, kib;
+  };
+  const Candidate candidates[] = {{4, 64}, {4, 1024}, {4, 4096}, {2, 0}};
+  std::unique_ptr<DevicePlan> best;
+  for (const Candidate& cand : candidates) {
+    mmr_plan_options o = base;
+    o.order = cand.order;
+    o.flags = (o.flags & 0xffu) | (cand.kib << 8);
+    auto alt = std::make_unique<DevicePlan>();
+    float ms = 0;
+    // a candidate that fails to build or to run (out of memory, say) is skipped: the default stays valid
+    int crc = make_device_plan(ctx, dp->plan.srcs, dp->plan.dsts, o, true, alt.get());
+    if (crc == MMR_OK) crc = time_plan(alt.get(), &ms);
+    if (crc == MMR_OK) {
+      timed += 1;
+      if (ms < 0.98f * best_ms) {  // only a clear win replaces the default
+        if (best) drop_bindings_of_plan(ctx, best.get());
+        best_ms = ms;
+        best = std::move(alt);
+        continue;
+      }
+    } else {
+      (void)hipGetLastError();
+    }
+    drop_bindings_of_plan(ctx, alt.get());
+  }
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  if (best) {  // the winner takes the default's place in the cache
+    drop_bindings_of_plan(ctx, dp);
+    drop_bindings_of_plan(ctx, best.get());
+    best->plan.stats.order_used = best->plan.options.order;
+    best->plan.options = base;  // still the plan of the context's options
+    ctx->plans[key] = std::move(best);
+    dp = ctx->plans[key].get();
+  }
+  dp->plan.stats.orders_timed = timed;
+  if (order_used) *order_used = dp->plan.stats.order_used;
   return MMR_OK;
 }
 
-// mmr_reshard_batch_static: the same argument checks, plan and kernels as reshard_locked, but the tables of the launch
-// go into this GPU's static scratch array (host plan -> pinned staging -> one stream-ordered copy) and nothing is
-// allocated on the device.  Layout in the array: pointer table, then the three chunk tables, each 256-byte aligned.
+// mmr_reshard_batch_static: the same argument checks, plan and kernels as reshard_locked, but every table of the
+// launch goes into this GPU's static scratch array (pinned staging -> one stream-ordered copy) and nothing is
+// allocated on the device.
 int reshard_static_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int n) {
   if (n == 0) return MMR_OK;
   if (int rc = use_device(ctx)) return rc;
   if (int rc = check_batch(ctx, srcs, dsts, n)) return rc;
-  std::vector<mmr_sharded_shape> sshapes(n), dshapes(n);
-  for (int a = 0; a < n; ++a) {
-    sshapes[a] = srcs[a]->shape;
-    dshapes[a] = dsts[a]->shape;
+  std::vector<mmr_sharded_shape> sshapes, dshapes;
+  shapes_of(srcs, dsts, n, &sshapes, &dshapes);
+  // host-side plans of their own (a cached DevicePlan may hold device tables; this path may not create any)
+  std::string key = "static:" + mmr::plan_key(sshapes.data(), dshapes.data(), n, ctx->options);
+  auto it = ctx->plans.find(key);
+  if (it == ctx->plans.end()) {
+    auto dp = std::make_unique<DevicePlan>();
+    if (int rc = make_device_plan(ctx, sshapes, dshapes, ctx->options, /*device_tables=*/false, dp.get())) return rc;
+    it = ctx->plans.emplace(key, std::move(dp)).first;
+    ctx->plan_lru.push_back(key);
+    ctx->stats.plans_cached = static_cast<int64_t>(ctx->plans.size());
   }
-  std::string key = mmr::plan_key(sshapes.data(), dshapes.data(), n, ctx->options);
-  auto it = ctx->static_plans.find(key);
-  if (it == ctx->static_plans.end()) {
-    auto plan = std::make_unique<mmr_plan>();
-    if (int rc = mmr::build_plan(sshapes.data(), dshapes.data(), n, ctx->options, plan.get())) return rc;
-    it = ctx->static_plans.emplace(std::move(key), std::move(plan)).first;
-  }
-  const mmr_plan& p = *it->second;
-  std::vector<TransposeRun> runs;
-  if (int rc = check_transposes(p, &runs)) return rc;
-  auto round_up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
-  const size_t ptr_bytes = static_cast<size_t>(p.n_slots) * sizeof(void*);
-  const size_t off16 = round_up(ptr_bytes);
-  const size_t off_generic = off16 + round_up(p.copy16.size() * sizeof(mmr_copy_chunk));
-  const size_t off_transposes = off_generic + round_up(p.generic.size() * sizeof(mmr_copy_chunk));
-  const size_t total = off_transposes + round_up(p.transposes.size() * sizeof(mmr_transpose_chunk));
-  if (total > MMR_STATIC_SCRATCH_BYTES)
+  const DevicePlan& dp = *it->second;
+  const BlockLayout l = layout_block(dp, /*with_chunk_tables=*/true);
+  if (l.total > MMR_STATIC_SCRATCH_BYTES)
     return fail(MMR_INVALID_ARGUMENT,
-                "the tables of this reshard take %zu bytes, the static scratch array holds %u: use mmr_reshard_batch", total,
+                "the tables of this reshard take %zu bytes, the static scratch array holds %u: use mmr_reshard_batch", l.total,
                 static_cast<unsigned>(MMR_STATIC_SCRATCH_BYTES));
   if (ctx->static_copy_pending) {  // the staging buffer is free again once the previous call's copy has read it
-    MMR_HIP(hipEventSynchronize(ctx->static_copied));
+    if (hipEventQuery(ctx->static_copied) != hipSuccess) {
+      ctx->stats.host_blocking_syncs += 1;
+      MMR_HIP(hipEventSynchronize(ctx->static_copied));
+    }
     ctx->static_copy_pending = false;
   }
-  void** ptrs = reinterpret_cast<void**>(ctx->static_staging);
-  for (int a = 0; a < n; ++a) {
-    size_t slot = static_cast<size_t>(p.slot_bases[a]);
-    for (int64_t k = 0; k < srcs[a]->side.dev_count; ++k) ptrs[slot++] = srcs[a]->tile(k);
-    for (int64_t k = 0; k < dsts[a]->side.dev_count; ++k) ptrs[slot++] = dsts[a]->tile(k);
-  }
-  if (!p.copy16.empty()) std::memcpy(ctx->static_staging + off16, p.copy16.data(), p.copy16.size() * sizeof(mmr_copy_chunk));
-  if (!p.generic.empty())
-    std::memcpy(ctx->static_staging + off_generic, p.generic.data(), p.generic.size() * sizeof(mmr_copy_chunk));
-  if (!p.transposes.empty())
-    std::memcpy(ctx->static_staging + off_transposes, p.transposes.data(), p.transposes.size() * sizeof(mmr_transpose_chunk));
+  std::vector<void*> ptrs;
+  collect_ptrs(dp.plan, srcs, dsts, n, &ptrs);
+  fill_block(dp, l, ptrs, true, ctx->static_staging);
   // stream-ordered: the copy waits for the kernels of the previous call on this stream, which still read the array
-  MMR_HIP(hipMemcpyAsync(ctx->static_scratch, ctx->static_staging, total, hipMemcpyHostToDevice, ctx->stream));
+  MMR_HIP(hipMemcpyAsync(ctx->static_scratch, ctx->static_staging, l.total, hipMemcpyHostToDevice, ctx->stream));
   MMR_HIP(hipEventRecord(ctx->static_copied, ctx->stream));
   ctx->static_copy_pending = true;
   ctx->stats.reshard_calls += 1;
-  char* base = ctx->static_scratch;
-  const int64_t launches = static_cast<int64_t>(runs.size()) + (p.copy16.empty() ? 0 : 1) + (p.generic.empty() ? 0 : 1);
-  if (int rc = launch_tables(ctx, p, reinterpret_cast<const mmr_copy_chunk*>(base + off16),
-                             reinterpret_cast<const mmr_copy_chunk*>(base + off_generic),
-                             reinterpret_cast<const mmr_transpose_chunk*>(base + off_transposes), runs,
-                             reinterpret_cast<void* const*>(base)))
+  const char* base = ctx->static_scratch;
+  if (int rc = launch_block(ctx, dp, base, l, reinterpret_cast<const mmr_copy_chunk*>(base + l.generic),
+                            reinterpret_cast<const mmr_transpose_chunk*>(base + l.transposes), true, true))
     return rc;
-  ctx->stats.kernel_launches += launches;
+  ctx->stats.kernel_launches += launches_of(&dp);
   return MMR_OK;
 }
 
@@ -493,7 +827,11 @@ void mmr_context_destroy(mmr_context* ctx) {
   if (!ctx) return;
   (void)hipSetDevice(ctx->device);
   (void)hipStreamSynchronize(ctx->stream);
-  for (auto& b : ctx->bindings) (void)hipFree(b.second->d_ptrs);
+  for (auto& b : ctx->bindings) {
+    (void)hipFree(b->d_block);
+    if (b->uploaded) (void)hipEventDestroy(b->uploaded);
+  }
+  ctx->bindings.clear();
   ctx->plans.clear();
   for (auto& s : ctx->stores) {
     (void)hipFree(s.second->base);
@@ -501,8 +839,13 @@ void mmr_context_destroy(mmr_context* ctx) {
   }
   for (auto& c : ctx->buffer_cache)
     for (auto& b : c.second) (void)hipFree(b.base);
+  for (auto& c : ctx->free_pool)
+    for (char* b : c.second) (void)hipFree(b);
+  for (auto& c : ctx->host_cache)
+    for (auto& b : c.second) (void)hipHostFree(b.base);
   (void)hipEventDestroy(ctx->t0);
   (void)hipEventDestroy(ctx->t1);
+  for (hipEvent_t e : ctx->laps) (void)hipEventDestroy(e);
   if (ctx->static_copied) (void)hipEventDestroy(ctx->static_copied);
   if (ctx->static_staging) (void)hipHostFree(ctx->static_staging);
   if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
@@ -518,15 +861,37 @@ int mmr_context_stream(mmr_context* ctx, void** hip_stream) {
 int mmr_context_set_plan_options(mmr_context* ctx, const mmr_plan_options* options) {
   if (!ctx) return fail(MMR_INVALID_ARGUMENT, "null context");
   std::lock_guard<std::mutex> lock(ctx->mu);
-  ctx->options = options ? *options : mmr_plan_options{};
-  // bindings point at plans built under the old options
-  for (auto& b : ctx->bindings) (void)hipFree(b.second->d_ptrs);
-  ctx->bindings.clear();
+  ctx->options = options ? *options : mmr_plan_options{};  // part of every plan's cache key
   return MMR_OK;
 }
 
-int mmr_store_create(mmr_context* ctx, const mmr_sharded_shape* shape, const char* name, uint32_t flags,
-                     mmr_store** out) {
+int mmr_context_set_flags(mmr_context* ctx, uint32_t flags) {
+  if (!ctx) return fail(MMR_INVALID_ARGUMENT, "null context");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  ctx->flags = flags;
+  return MMR_OK;
+}
+
+int mmr_context_clear_plans(mmr_context* ctx) {
+  if (!ctx) return fail(MMR_INVALID_ARGUMENT, "null context");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  if (int rc = use_device(ctx)) return rc;
+  if (int rc = refuse_capture(ctx, "mmr_context_clear_plans")) return rc;
+  if (int rc = blocking_sync(ctx)) return rc;
+  for (auto& b : ctx->bindings) {
+    (void)hipFree(b->d_block);
+    if (b->uploaded) (void)hipEventDestroy(b->uploaded);
+  }
+  ctx->bindings.clear();
+  ctx->plans.clear();
+  ctx->plan_lru.clear();
+  ctx->stats.plans_cached = 0;
+  ctx->stats.bindings_cached = 0;
+  return MMR_OK;
+}
+
+int mmr_store_create_ex(mmr_context* ctx, const mmr_sharded_shape* shape, const char* name, uint32_t flags,
+                        int64_t min_cache_size, mmr_store** out) {
   if (!ctx || !shape || !out) return fail(MMR_INVALID_ARGUMENT, "null argument");
   std::lock_guard<std::mutex> lock(ctx->mu);
   if (int rc = use_device(ctx)) return rc;
@@ -540,24 +905,54 @@ int mmr_store_create(mmr_context* ctx, const mmr_sharded_shape* shape, const cha
   s->bytes = s->pitch * static_cast<size_t>(s->side.dev_count);
   bool reused = false;
   if (flags & MMR_STORE_FROM_CACHE) {
-    auto it = ctx->buffer_cache.find(s->shape_key);
-    if (it != ctx->buffer_cache.end() && !it->second.empty()) {
-      s->base = it->second.back().base;
-      it->second.pop_back();
+    std::vector<CachedBuffer>& parked = ctx->buffer_cache[s->shape_key];
+    if (!parked.empty()) {
+      s->base = parked.back().base;
+      parked.pop_back();
       ctx->stats.cache_hits += 1;
       reused = true;
     }
   }
   if (!reused) {
-    MMR_HIP(hipMalloc(reinterpret_cast<void**>(&s->base), s->bytes));
-    MMR_HIP(hipMemsetAsync(s->base, 0, s->bytes, ctx->stream));
-    account_alloc(ctx, static_cast<int64_t>(s->bytes));
+    auto pooled = ctx->free_pool.find(s->bytes);
+    if (pooled != ctx->free_pool.end() && !pooled->second.empty()) {
+      s->base = pooled->second.back();
+      pooled->second.pop_back();
+      ctx->free_pool_bytes -= s->bytes;
+      ctx->stats.pool_hits += 1;
+    } else {
+      if (int rc = refuse_capture(ctx, "creating a store that needs new device memory")) return rc;
+      if (int rc = device_alloc(ctx, reinterpret_cast<void**>(&s->base), s->bytes)) return rc;
+      account_alloc(ctx, static_cast<int64_t>(s->bytes));
+    }
+    if (!(flags & MMR_STORE_UNINITIALIZED)) {
+      if (int rc = refuse_capture(ctx, "zero-filling a new store")) return rc;
+      MMR_HIP(hipMemsetAsync(s->base, 0, s->bytes, ctx->stream));
+    }
+    if (flags & MMR_STORE_FROM_CACHE) {
+      // ArrayCache::Get(shape, min_cache_size): the cache of this descriptor holds at least that many buffers
+      std::vector<CachedBuffer>& parked = ctx->buffer_cache[s->shape_key];
+      for (int64_t extra = 1; extra < min_cache_size; ++extra) {
+        char* more = nullptr;
+        if (int rc = device_alloc(ctx, reinterpret_cast<void**>(&more), s->bytes)) return rc;
+        account_alloc(ctx, static_cast<int64_t>(s->bytes));
+        if (!(flags & MMR_STORE_UNINITIALIZED)) MMR_HIP(hipMemsetAsync(more, 0, s->bytes, ctx->stream));
+        parked.push_back(CachedBuffer{more, s->bytes});
+      }
+    }
   }
   s->id = g_next_store_id.fetch_add(1);
+  s->ordinal = ctx->next_ordinal++;
+  hash_op(ctx, 1 /* CreateStore */, {static_cast<uint64_t>(s->ordinal)}, &s->shape_key);
   ctx->stats.stores_live += 1;
   *out = s.get();
   ctx->stores.emplace(s->id, std::move(s));
   return MMR_OK;
+}
+
+int mmr_store_create(mmr_context* ctx, const mmr_sharded_shape* shape, const char* name, uint32_t flags,
+                     mmr_store** out) {
+  return mmr_store_create_ex(ctx, shape, name, flags, 1, out);
 }
 
 int mmr_store_free(mmr_context* ctx, mmr_store* store, int32_t keep_in_cache) {
@@ -565,17 +960,23 @@ int mmr_store_free(mmr_context* ctx, mmr_store* store, int32_t keep_in_cache) {
   std::lock_guard<std::mutex> lock(ctx->mu);
   if (int rc = check_store(ctx, store, "freed")) return rc;
   if (int rc = use_device(ctx)) return rc;
-  drop_bindings_of(ctx, store->id);
+  hash_op(ctx, 3 /* Free */, {static_cast<uint64_t>(store->ordinal), static_cast<uint64_t>(keep_in_cache != 0)});
   if (store->host) {
-    MMR_HIP(hipHostFree(store->host));
-    ctx->stats.host_bytes_allocated -= static_cast<int64_t>(store->bytes);
+    // the pinned buffer goes back to the host cache (a copy still in flight on the stream is ordered before its next use)
+    ctx->host_cache[store->shape_key].push_back(CachedBuffer{store->host, store->bytes});
   } else if (!store->adopted.empty()) {
     // caller-owned buffers: in-flight work on them must finish before the caller may reuse them
-    MMR_HIP(hipStreamSynchronize(ctx->stream));
+    if (int rc = refuse_capture(ctx, "freeing a store of adopted buffers")) return rc;
+    if (int rc = blocking_sync(ctx)) return rc;
   } else if (keep_in_cache) {
     ctx->buffer_cache[store->shape_key].push_back(CachedBuffer{store->base, store->bytes});
+  } else if (ctx->free_pool_bytes + store->bytes <= kFreePoolLimit) {
+    ctx->free_pool[store->bytes].push_back(store->base);  // back to the allocator's pool: no device-wide wait
+    ctx->free_pool_bytes += store->bytes;
   } else {
-    MMR_HIP(hipFree(store->base));
+    if (int rc = refuse_capture(ctx, "freeing device memory")) return rc;
+    MMR_HIP(hipFree(store->base));  // waits for the device
+    ctx->stats.host_blocking_syncs += 1;
     ctx->stats.bytes_allocated -= static_cast<int64_t>(store->bytes);
   }
   ctx->stats.stores_live -= 1;
@@ -587,6 +988,7 @@ int mmr_clear_store_cache(mmr_context* ctx) {
   if (!ctx) return fail(MMR_INVALID_ARGUMENT, "null context");
   std::lock_guard<std::mutex> lock(ctx->mu);
   if (int rc = use_device(ctx)) return rc;
+  if (int rc = refuse_capture(ctx, "mmr_clear_store_cache")) return rc;
   for (auto& c : ctx->buffer_cache) {
     for (auto& b : c.second) {
       MMR_HIP(hipFree(b.base));
@@ -594,6 +996,24 @@ int mmr_clear_store_cache(mmr_context* ctx) {
     }
   }
   ctx->buffer_cache.clear();
+  for (auto& c : ctx->free_pool)
+    for (char* b : c.second) {
+      MMR_HIP(hipFree(b));
+      ctx->stats.bytes_allocated -= static_cast<int64_t>(c.first);
+    }
+  ctx->free_pool.clear();
+  ctx->free_pool_bytes = 0;
+  bool any_host = false;
+  for (auto& c : ctx->host_cache) any_host |= !c.second.empty();
+  if (any_host)
+    if (int rc = blocking_sync(ctx)) return rc;  // a reload may still be reading one of them
+  for (auto& c : ctx->host_cache) {
+    for (auto& b : c.second) {
+      MMR_HIP(hipHostFree(b.base));
+      ctx->stats.host_bytes_allocated -= static_cast<int64_t>(b.bytes);
+    }
+  }
+  ctx->host_cache.clear();
   return MMR_OK;
 }
 
@@ -607,6 +1027,7 @@ int mmr_store_assemble(mmr_context* ctx, mmr_store* store, int64_t device, const
   if (size > static_cast<size_t>(store->side.shard_bytes))
     return fail(MMR_INVALID_ARGUMENT, "shard of %zu bytes does not fit the %lld-byte buffer of store %lld", size,
                 (long long)store->side.shard_bytes, (long long)store->id);
+  hash_op(ctx, 4 /* AssembleShards */, {static_cast<uint64_t>(store->ordinal), static_cast<uint64_t>(device), size});
   if (size == 0) return MMR_OK;
   if (!data) return fail(MMR_INVALID_ARGUMENT, "null shard data");
   if (int rc = use_device(ctx)) return rc;
@@ -616,7 +1037,7 @@ int mmr_store_assemble(mmr_context* ctx, mmr_store* store, int64_t device, const
                              : data_on_device == 0 ? hipMemcpyHostToDevice
                                                    : hipMemcpyDefault;  // the runtime looks the pointer up
   if (store->offloaded()) return fail(MMR_INVALID_ARGUMENT, "store %lld is offloaded to host memory", (long long)store->id);
-  if (data_on_device == 2 && size >= (1u << 20)) {  // worth asking the runtime where the pointer lives
+  if (data_on_device == 2) {  // ask the runtime where the pointer lives: a device-resident shard needs no host wait
     hipPointerAttribute_t attr{};
     if (hipPointerGetAttributes(&attr, data) == hipSuccess) {
       if (attr.type == hipMemoryTypeDevice && attr.device == ctx->device) data_on_device = 1;
@@ -636,8 +1057,11 @@ int mmr_store_assemble(mmr_context* ctx, mmr_store* store, int64_t device, const
                              hipMemcpyDeviceToDevice, ctx->stream));
     return MMR_OK;
   }
+  if (data_on_device != 1)
+    if (int rc = refuse_capture(ctx, "assembling a shard from host memory")) return rc;
   MMR_HIP(hipMemcpyAsync(store->tile(k), data, size, kind, ctx->stream));
-  if (data_on_device != 1) MMR_HIP(hipStreamSynchronize(ctx->stream));  // host data is consumed before returning
+  if (data_on_device != 1)
+    if (int rc = blocking_sync(ctx)) return rc;  // host data is consumed before returning
   return MMR_OK;
 }
 
@@ -667,14 +1091,14 @@ int mmr_store_read_shard(mmr_context* ctx, mmr_store* store, int64_t device, voi
     return fail(MMR_INVALID_ARGUMENT, "read of %zu bytes exceeds the %lld-byte shard", size,
                 (long long)store->side.shard_bytes);
   if (int rc = use_device(ctx)) return rc;
+  if (int rc = refuse_capture(ctx, "reading a shard back")) return rc;
   if (store->offloaded()) {
-    MMR_HIP(hipStreamSynchronize(ctx->stream));
+    if (int rc = blocking_sync(ctx)) return rc;  // the copy to the pinned buffer is done after this
     std::memcpy(host_dst, store->host + static_cast<size_t>(k) * store->pitch, size);
     return MMR_OK;
   }
   if (size) MMR_HIP(hipMemcpyAsync(host_dst, store->tile(k), size, hipMemcpyDeviceToHost, ctx->stream));
-  MMR_HIP(hipStreamSynchronize(ctx->stream));
-  return MMR_OK;
+  return blocking_sync(ctx);
 }
 
 int mmr_store_has_shard(const mmr_store* store, int64_t device, int32_t* out) {
@@ -711,6 +1135,8 @@ int mmr_store_adopt(mmr_context* ctx, const mmr_sharded_shape* shape, const char
   s->pitch = static_cast<size_t>(s->side.shard_bytes);
   s->bytes = 0;
   s->id = g_next_store_id.fetch_add(1);
+  s->ordinal = ctx->next_ordinal++;
+  hash_op(ctx, 5 /* adopt */, {static_cast<uint64_t>(s->ordinal)}, &s->shape_key);
   ctx->stats.stores_live += 1;
   *out = s.get();
   ctx->stores.emplace(s->id, std::move(s));
@@ -724,16 +1150,25 @@ int mmr_store_offload(mmr_context* ctx, mmr_store* store) {
   if (store->offloaded()) return MMR_OK;
   if (!store->adopted.empty()) return fail(MMR_INVALID_ARGUMENT, "store %lld lives in caller-owned buffers", (long long)store->id);
   if (int rc = use_device(ctx)) return rc;
-  // pinned host memory is allocated, never registered after the fact
-  MMR_HIP(hipHostMalloc(reinterpret_cast<void**>(&store->host), store->bytes, hipHostMallocDefault));
+  hash_op(ctx, 6 /* OffloadDtoH */, {static_cast<uint64_t>(store->ordinal)});
+  // a pinned buffer from the host cache of this descriptor, else a new one (allocated pinned, never registered
+  // after the fact)
+  std::vector<CachedBuffer>& pool = ctx->host_cache[store->shape_key];
+  if (!pool.empty()) {
+    store->host = pool.back().base;
+    pool.pop_back();
+    ctx->stats.host_cache_hits += 1;
+  } else {
+    if (int rc = refuse_capture(ctx, "offloading a store that needs a new pinned buffer")) return rc;
+    MMR_HIP(hipHostMalloc(reinterpret_cast<void**>(&store->host), store->bytes, hipHostMallocDefault));
+    ctx->stats.host_bytes_allocated += static_cast<int64_t>(store->bytes);
+    ctx->stats.host_bytes_high_watermark = std::max(ctx->stats.host_bytes_high_watermark, ctx->stats.host_bytes_allocated);
+  }
+  // ordered on the stream behind whatever produced the store (the `pipelined` stores of OffloadDtoH included); the
+  // device buffer goes to the device cache at once: its next user is ordered on the same stream behind this copy
   MMR_HIP(hipMemcpyAsync(store->host, store->base, store->bytes, hipMemcpyDeviceToHost, ctx->stream));
-  MMR_HIP(hipStreamSynchronize(ctx->stream));
-  drop_bindings_of(ctx, store->id);
-  MMR_HIP(hipFree(store->base));
+  ctx->buffer_cache[store->shape_key].push_back(CachedBuffer{store->base, store->bytes});
   store->base = nullptr;
-  ctx->stats.bytes_allocated -= static_cast<int64_t>(store->bytes);
-  ctx->stats.host_bytes_allocated += static_cast<int64_t>(store->bytes);
-  ctx->stats.host_bytes_high_watermark = std::max(ctx->stats.host_bytes_high_watermark, ctx->stats.host_bytes_allocated);
   return MMR_OK;
 }
 
@@ -743,13 +1178,21 @@ int mmr_store_reload(mmr_context* ctx, mmr_store* store) {
   if (int rc = check_store(ctx, store, "reloaded")) return rc;
   if (!store->offloaded()) return MMR_OK;
   if (int rc = use_device(ctx)) return rc;
-  MMR_HIP(hipMalloc(reinterpret_cast<void**>(&store->base), store->bytes));
-  account_alloc(ctx, static_cast<int64_t>(store->bytes));
+  hash_op(ctx, 7 /* OffloadHtoD */, {static_cast<uint64_t>(store->ordinal)});
+  std::vector<CachedBuffer>& parked = ctx->buffer_cache[store->shape_key];
+  if (!parked.empty()) {
+    store->base = parked.back().base;
+    parked.pop_back();
+    ctx->stats.cache_hits += 1;
+  } else {
+    if (int rc = refuse_capture(ctx, "reloading a store that needs new device memory")) return rc;
+    if (int rc = device_alloc(ctx, reinterpret_cast<void**>(&store->base), store->bytes)) return rc;
+    account_alloc(ctx, static_cast<int64_t>(store->bytes));
+  }
   MMR_HIP(hipMemcpyAsync(store->base, store->host, store->bytes, hipMemcpyHostToDevice, ctx->stream));
-  MMR_HIP(hipStreamSynchronize(ctx->stream));  // the pinned buffer is released right away
-  MMR_HIP(hipHostFree(store->host));
+  // the pinned buffer goes to the host cache at once: the next offload into it is ordered behind this copy
+  ctx->host_cache[store->shape_key].push_back(CachedBuffer{store->host, store->bytes});
   store->host = nullptr;
-  ctx->stats.host_bytes_allocated -= static_cast<int64_t>(store->bytes);
   return MMR_OK;
 }
 
@@ -797,6 +1240,12 @@ int mmr_reshard_batch_static(mmr_context* ctx, mmr_store* const* srcs, mmr_store
   if (!ctx || n < 0 || (n > 0 && (!srcs || !dsts))) return fail(MMR_INVALID_ARGUMENT, "bad batch arguments");
   std::lock_guard<std::mutex> lock(ctx->mu);
   return reshard_static_locked(ctx, srcs, dsts, n);
+}
+
+int mmr_reshard_tune(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int32_t n, int64_t* order_used) {
+  if (!ctx || n <= 0 || !srcs || !dsts) return fail(MMR_INVALID_ARGUMENT, "bad batch arguments");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  return tune_locked(ctx, srcs, dsts, n, order_used);
 }
 
 int mmr_reshard_validate(mmr_context* ctx, mmr_store* src, mmr_store* dst) {
@@ -847,6 +1296,30 @@ int mmr_timer_stop(mmr_context* ctx, float* milliseconds) {
   return MMR_OK;
 }
 
+int mmr_timer_lap(mmr_context* ctx) {
+  if (!ctx) return fail(MMR_INVALID_ARGUMENT, "null context");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  if (ctx->laps_used == ctx->laps.size()) {
+    hipEvent_t e = nullptr;
+    MMR_HIP(hipEventCreate(&e));
+    ctx->laps.push_back(e);
+  }
+  MMR_HIP(hipEventRecord(ctx->laps[ctx->laps_used], ctx->stream));
+  ctx->laps_used += 1;
+  return MMR_OK;
+}
+
+int mmr_timer_laps(mmr_context* ctx, float* milliseconds, int32_t capacity, int32_t* count) {
+  if (!ctx || !count || (capacity > 0 && !milliseconds)) return fail(MMR_INVALID_ARGUMENT, "null argument");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  const size_t n = ctx->laps_used > 0 ? ctx->laps_used - 1 : 0;
+  if (ctx->laps_used > 0) MMR_HIP(hipEventSynchronize(ctx->laps[ctx->laps_used - 1]));
+  *count = static_cast<int32_t>(std::min<size_t>(n, static_cast<size_t>(std::max(capacity, 0))));
+  for (int32_t i = 0; i < *count; ++i) MMR_HIP(hipEventElapsedTime(&milliseconds[i], ctx->laps[i], ctx->laps[i + 1]));
+  ctx->laps_used = 0;
+  return MMR_OK;
+}
+
 int mmr_context_get_stats(mmr_context* ctx, mmr_context_stats* out) {
   if (!ctx || !out) return fail(MMR_INVALID_ARGUMENT, "null argument");
   std::lock_guard<std::mutex> lock(ctx->mu);
@@ -858,13 +1331,12 @@ int mmr_reshard_batch_plan_stats(mmr_context* ctx, mmr_store* const* srcs, mmr_s
                                  mmr_plan_stats* out) {
   if (!ctx || !out || n <= 0 || !srcs || !dsts) return fail(MMR_INVALID_ARGUMENT, "bad arguments");
   std::lock_guard<std::mutex> lock(ctx->mu);
-  std::vector<mmr_sharded_shape> s(static_cast<size_t>(n)), d(static_cast<size_t>(n));
   for (int a = 0; a < n; ++a) {
     if (int rc = check_store(ctx, srcs[a], "source")) return rc;
     if (int rc = check_store(ctx, dsts[a], "destination")) return rc;
-    s[a] = srcs[a]->shape;
-    d[a] = dsts[a]->shape;
   }
+  std::vector<mmr_sharded_shape> s, d;
+  shapes_of(srcs, dsts, n, &s, &d);
   if (int rc = use_device(ctx)) return rc;
   DevicePlan* dp = nullptr;
   if (int rc = get_plan(ctx, s, d, &dp)) return rc;

@@ -1,6 +1,8 @@
 // See hip_execute_context.h.
 #include "hip_execute_context.h"
 
+#include <hip/hip_runtime_api.h>
+
 #include <stdexcept>
 
 namespace mmr {
@@ -49,6 +51,21 @@ int64_t ShardSize(const ShardedShape& shape) {
   int64_t bytes = 0;
   check(mmr_shard_bytes(&p, &bytes), "ShardSize");
   return bytes;
+}
+
+MultiMeshStream::~MultiMeshStream() {
+  if (event_) (void)hipEventDestroy(static_cast<hipEvent_t>(event_));
+}
+
+void* MultiMeshStream::RecordEvent() {
+  if (!event_) {
+    hipEvent_t e = nullptr;
+    if (hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess) raise("MultiMeshStream: hipEventCreate failed");
+    event_ = e;
+  }
+  if (hipEventRecord(static_cast<hipEvent_t>(event_), static_cast<hipStream_t>(stream_)) != hipSuccess)
+    raise("MultiMeshStream: hipEventRecord failed");
+  return event_;
 }
 
 // One sharded array; freed when the last handle of the last device lets go.
@@ -124,7 +141,9 @@ StoreHandle HipExecuteContext::CreateStore(int64_t local_device_id, int64_t glob
     shared->shape = shape;
     mmr_sharded_shape pod = shape.ToPod();
     const char* name = config.name.has_value() ? config.name->c_str() : nullptr;
-    int rc = mmr_store_create(ctx_, &pod, name, config.allocate_from_cache ? MMR_STORE_FROM_CACHE : 0, &shared->store);
+    const uint32_t flags = (config.allocate_from_cache ? MMR_STORE_FROM_CACHE : 0u) |
+                           (config.uninitialized ? MMR_STORE_UNINITIALIZED : 0u);
+    int rc = mmr_store_create_ex(ctx_, &pod, name, flags, config.min_cache_size.value_or(1), &shared->store);
     if (rc != MMR_OK) {
       in_flight_["CreateStore"].erase(seq);
       next_seq_["CreateStore"][local_device_id]--;
@@ -147,7 +166,8 @@ StoreHandle HipExecuteContext::CreateStore(int64_t local_device_id, int64_t glob
 }
 
 StoreHandle HipExecuteContext::AssembleShards(int64_t local_device_id, int64_t global_device_id, ShardedShape shape,
-                                              Shard shard, std::optional<StoreHandle> existing_store) {
+                                              Shard shard, std::shared_ptr<MultiMeshStream> stream,
+                                              std::optional<StoreHandle> existing_store) {
   StoreHandle output =
       existing_store.has_value() ? *std::move(existing_store) : CreateStore(local_device_id, global_device_id, shape);
   require_live(output, "AssembleShards");
@@ -155,6 +175,9 @@ StoreHandle HipExecuteContext::AssembleShards(int64_t local_device_id, int64_t g
   FlushLocked();
   // across(shape.sharding.devices).if_on(p): only a member device copies its shard
   if (shape.sharding.devices.Contains(global_device_id)) {
+    // behind the producer of the native shard, on the device (zuku_execute_context_impl.cc:410-414 issues the copy on
+    // the producer's own stream)
+    if (stream && stream->hip_stream()) check(mmr_context_wait_event(ctx_, stream->RecordEvent()), "AssembleShards");
     check(mmr_store_assemble(ctx_, output.impl->array->store, global_device_id, shard.data, shard.size, 2),
           "AssembleShards");
   }
@@ -224,6 +247,12 @@ void HipExecuteContext::Flush() {
   FlushLocked();
 }
 
+void HipExecuteContext::SetCheckInvariants(bool on) {
+  std::lock_guard<std::mutex> lock(mu_);
+  FlushLocked();
+  check(mmr_context_set_flags(ctx_, on ? MMR_CHECK_INVARIANTS : 0u), "SetCheckInvariants");
+}
+
 void HipExecuteContext::SetDeferReshards(bool defer) {
   std::lock_guard<std::mutex> lock(mu_);
   FlushLocked();
@@ -261,10 +290,11 @@ void HipExecuteContext::Free(int64_t local_device_id, StoreHandle handle, bool k
   if (!handle.impl) return;
   std::lock_guard<std::mutex> lock(mu_);
   if (!handle.impl->array) return;  // already freed through another copy of this handle
-  // As in the reference (zuku_execute_context_impl.cc:509-514) the array is taken
-  // out of the shared impl, so every copy of this device's handle lets go; the
-  // buffers go back to the cache or the allocator when the last device has freed.
-  handle.impl->array->keep_in_cache = keep_in_cache;
+  // As in the reference (zuku_execute_context_impl.cc:504-515): with keep_in_cache the array is moved out of the shared
+  // impl into the cache, so every copy of this device's handle lets go (the buffers are parked once the last device has
+  // freed); without it only the copy passed by value is dropped and the array lives on for every other copy.
+  if (!keep_in_cache) return;
+  handle.impl->array->keep_in_cache = true;
   handle.impl->array.reset();
 }
 
@@ -382,7 +412,9 @@ std::vector<std::vector<StoreHandle>> ReshardSchedule::Execute(
     const Store& out = op.op.output;
     if (out.type != Store::Type::ROOT || root_stores[0][out.index].impl) continue;
     for (size_t i = 0; i < n; ++i)
-      root_stores[i][out.index] = ctx.CreateStore(devices[i], devices[i], out.sharded_shape, {.name = out.name});
+      // written entirely by the reshard that produces it (pad included): no zero fill
+      root_stores[i][out.index] =
+          ctx.CreateStore(devices[i], devices[i], out.sharded_shape, {.name = out.name, .uninitialized = true});
   }
   if (cached_temporary_stores_.empty()) {
     cached_temporary_stores_.resize(n);

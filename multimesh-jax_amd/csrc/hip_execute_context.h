@@ -108,7 +108,24 @@ struct Shard {
 struct CreateStoreConfig {
   std::optional<std::string> name{std::nullopt};
   bool allocate_from_cache{false};
-  std::optional<int64_t> min_cache_size{std::nullopt};
+  std::optional<int64_t> min_cache_size{std::nullopt};  // -> mmr_store_create_ex
+  bool uninitialized{false};  // extension: skip the zero fill (the store is a reshard's output: every byte is written)
+};
+
+// MultiMeshStream (mm_computation.h:131-149): the stream a native shard's producer runs on.  The reference issues the
+// assemble copy on it (zuku_execute_context_impl.cc:405-415); here the copy runs on the context's stream and is ordered
+// behind the producer's work by an event, without blocking the host.
+class MultiMeshStream {
+ public:
+  explicit MultiMeshStream(void* hip_stream) : stream_(hip_stream) {}
+  ~MultiMeshStream();
+  void* hip_stream() const { return stream_; }
+  // Records the producer's progress so far; returns the hipEvent_t (owned by this object).
+  void* RecordEvent();
+
+ private:
+  void* stream_;
+  void* event_{nullptr};
 };
 
 // store_handle_fwd.h:15-19, store_handle.h:16-20
@@ -141,8 +158,10 @@ class HipExecuteContext {
 
   StoreHandle CreateStore(int64_t local_device_id, int64_t global_device_id, ShardedShape shape,
                           CreateStoreConfig config = {});
-  // Shard.data: device or host memory (the runtime tells which).
+  // Shard.data: device or host memory (the runtime tells which).  stream: where the shard's producer runs (may be
+  // null: the shard is ready); the copy is ordered behind it on the device, the host does not wait.
   StoreHandle AssembleShards(int64_t local_device_id, int64_t global_device_id, ShardedShape shape, Shard shard,
+                             std::shared_ptr<MultiMeshStream> stream = nullptr,
                              std::optional<StoreHandle> existing_store = std::nullopt);
   void Reshard(int64_t local_device_id, int64_t global_device_id, const StoreHandle& src, const StoreHandle& dst);
   void* SliceLocalShard(int64_t local_device_id, const StoreHandle& handle);
@@ -175,6 +194,10 @@ class HipExecuteContext {
   // Flush() before it enqueues a task.  Argument errors are still raised by the Reshard call that causes them.
   void Flush();
   void SetDeferReshards(bool defer);
+  // The reference's mock keeps invariants every C++ test of the plugin runs under (mm_mock_mm_xla.cc:259-262 rolling
+  // hash of the operation stream, :347-369 every operand has a tile on each of its devices): kept here as a
+  // checking mode; Stats().operation_hash is equal between two runs that issue the same operations.
+  void SetCheckInvariants(bool on);
 
   // Not part of the reference interface: inspection for tests and benchmarks (both flush first).
   mmr_context* raw() {

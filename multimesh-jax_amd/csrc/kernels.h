@@ -6,18 +6,29 @@
 #include <hip/hip_runtime_api.h>
 
 #include "mmreshard.h"
+#include "group_ops.h"
 
 namespace mmr {
 
 // Flat device-to-device copy; both pointers and the size must be multiples of 16 (hipErrorInvalidValue otherwise).
 hipError_t launch_flat_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);
-// Chunks whose offsets, strides and widths are all multiples of 16 bytes.
+// Copy groups (every offset, stride and width a multiple of 16 bytes) of a bound table: n workgroups, one per
+// chunk, each decoding its chunk from the table.  d_hints: the group of the first chunk of every block of 64 chunks.
 // xcd_mode: 0/1 = chunk i runs as workgroup i (the hardware deals consecutive
 // workgroups round-robin over the 8 XCDs); 2 = each XCD takes a contiguous
 // eighth of the table; G >= 16 = runs of G consecutive chunks share an XCD (and
 // so an L2), runs dealt round-robin.
-hipError_t launch_copy16(const mmr_copy_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
-                         hipStream_t stream);
+// starts: host array of every group's first chunk (or null); tables of up to kMaxDirectGroups groups get it by value.
+hipError_t launch_copy_groups(const CopyGroup* d_groups, uint32_t n_groups, const CopyPiece* d_pieces,
+                              const uint32_t* d_hints, const uint32_t* starts, int64_t n, uint32_t xcd_mode,
+                              hipStream_t stream);
+// The same for a table small enough to travel in the kernel's argument block.
+hipError_t launch_copy_groups_inline(const InlineCopyTable& table, uint32_t xcd_mode, hipStream_t stream);
+// Span groups (ragged rows into dense destination tiles), staged through LDS.
+hipError_t launch_spans(const SpanGroup* d_groups, uint32_t n_groups, const SpanMember* d_members,
+                        const SpanPiece* d_pieces, const uint32_t* d_hints, int64_t n, uint32_t xcd_mode,
+                        hipStream_t stream);
+hipError_t launch_spans_inline(const InlineSpanTable& table, uint32_t xcd_mode, hipStream_t stream);
 // Chunks of any alignment (chunk.align picks the access width).
 hipError_t launch_copy_generic(const mmr_copy_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
                                hipStream_t stream);

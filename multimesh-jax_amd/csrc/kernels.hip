@@ -17,6 +17,7 @@
 #include <mutex>
 
 #include "chunk_ops.h"
+#include "group_ops.h"
 #include "kernels.h"
 
 namespace mmr {
@@ -74,6 +75,21 @@ struct DeviceMem {
   static __device__ __forceinline__ uintptr_t caddr(cptr p) { return reinterpret_cast<uintptr_t>(p); }
 };
 
+// LDS accesses of the span kernel.  gfx950 takes a 16-byte LDS access at any byte address (the compiler emits a single
+// ds_write_b128 for the aligned(1) type below).
+struct DeviceLds {
+  static __device__ __forceinline__ void store16u(uint8_t* p, V16 v) {
+    typedef u32x4 __attribute__((aligned(1))) u4u;
+    *reinterpret_cast<u4u*>(p) = u32x4{v.x, v.y, v.z, v.w};
+  }
+  static __device__ __forceinline__ void store8(uint8_t* p, uint8_t v) { *p = v; }
+  static __device__ __forceinline__ V16 load16(const uint8_t* p) {
+    const u32x4 v = *reinterpret_cast<const u32x4*>(p);
+    return V16{v.x, v.y, v.z, v.w};
+  }
+  static __device__ __forceinline__ uint8_t load8(const uint8_t* p) { return *p; }
+};
+
 __device__ __forceinline__ gchar* slot_base(void* const* __restrict__ ptrs, uint32_t slot, uint64_t off) {
   return (gchar*)(static_cast<char*>(ptrs[slot])) + off;
 }
@@ -85,16 +101,86 @@ __device__ __forceinline__ gchar* slot_base(void* const* __restrict__ ptrs, uint
 #ifndef MMR_COPY16_NT_LOADS
 #define MMR_COPY16_NT_LOADS true
 #endif
+#ifndef MMR_SPAN_UNROLL
+#define MMR_SPAN_UNROLL 2
+#endif
 
+// Copy groups: the workgroup works its chunk out from the group table (bound: absolute addresses).  `groups` and
+// `pieces` are wave-uniform reads (scalar loads); the records are taken by value so that their loads leave together.
 template <int THREADS, int UNROLL>
-__global__ __launch_bounds__(THREADS) void mmr_copy16_kernel(const mmr_copy_chunk* __restrict__ chunks, uint32_t n,
-                                                             void* const* __restrict__ ptrs, uint32_t xcd_group) {
+__device__ __forceinline__ void copy_group_chunk(const CopyGroup* __restrict__ groups, const CopyPiece* __restrict__ pieces,
+                                                 uint32_t gi, uint32_t ci) {
+  const CopyGroup g = groups[gi];
+  const DecodedCopy d = decode_copy(g, ci - g.first_chunk);
+  const CopyPiece p = pieces[d.piece];
+  const mmr_copy_chunk c = copy_chunk_of(g, p, d);
+  gchar* dst = (gchar*)(c.dst_off);
+  gcchar* src = c.src_slot == MMR_SLOT_FILL ? dst : (gcchar*)(c.src_off);  // never read when filling
+  copy_group_rows<DeviceMem<MMR_COPY16_NT_LOADS, true>, THREADS, UNROLL>(g, p, c, src, dst, threadIdx.x);
+}
+
+// DIRECT: the table has at most kMaxDirectGroups groups and `starts` holds their first chunks (no hint lookup).
+template <int THREADS, int UNROLL, bool DIRECT>
+__global__ __launch_bounds__(THREADS) void mmr_copy16_kernel(const CopyGroup* __restrict__ groups, uint32_t n_groups,
+                                                             const CopyPiece* __restrict__ pieces,
+                                                             const uint32_t* __restrict__ hints, uint32_t n,
+                                                             uint32_t xcd_group, const GroupStarts starts) {
   const uint32_t ci = chunk_index(blockIdx.x, xcd_group);
   if (ci >= n) return;
-  const mmr_copy_chunk c = chunks[ci];
-  gchar* dst = slot_base(ptrs, c.dst_slot, c.dst_off);
-  gcchar* src = c.src_slot == MMR_SLOT_FILL ? dst : slot_base(ptrs, c.src_slot, c.src_off);  // never read when filling
-  copy16_chunk<DeviceMem<MMR_COPY16_NT_LOADS, true>, THREADS, UNROLL>(c, src, dst, threadIdx.x);
+  const uint32_t gi = DIRECT ? find_group_direct(starts, ci) : find_group(groups, n_groups, hints, ci);
+  copy_group_chunk<THREADS, UNROLL>(groups, pieces, gi, ci);
+}
+
+// The same with the whole table in the kernel's argument block (nothing in device memory to look up or to keep alive).
+template <int THREADS, int UNROLL>
+__global__ __launch_bounds__(THREADS) void mmr_copy16_inline_kernel(const InlineCopyTable table, uint32_t xcd_group) {
+  const uint32_t ci = chunk_index(blockIdx.x, xcd_group);
+  if (ci >= table.n_chunks) return;
+  copy_group_chunk<THREADS, UNROLL>(table.groups, table.pieces, find_group(table.groups, table.n_groups, nullptr, ci), ci);
+}
+
+// 16 readable bytes for the loads of span items that need none.
+__device__ __align__(16) const uint32_t span_safe_bytes[4] = {0, 0, 0, 0};
+
+template <int THREADS, int UNROLL>
+__device__ __forceinline__ void span_chunk(const SpanGroup* __restrict__ groups, uint32_t n_groups,
+                                           const SpanMember* __restrict__ members, const SpanPiece* __restrict__ pieces,
+                                           const uint32_t* __restrict__ hints, uint32_t ci, uint8_t* lds) {
+  typedef DeviceMem<false, true> M;  // cacheable loads: neighbouring tiles' spans share source lines
+  const uint32_t gi = find_group(groups, n_groups, hints, ci);
+  const SpanGroup g = groups[gi];
+  uint32_t member, lm;
+  deinterleave(g.il, ci - g.first_chunk, &member, &lm);
+  const SpanMember m = members[g.first_member + member];
+  uint64_t x0;
+  uint32_t len;
+  span_range(g, lm, &x0, &len);
+  gchar* dst = (gchar*)(m.dst + x0);
+  const uint32_t a = static_cast<uint32_t>(m.dst + x0) & 15u;
+  gcchar* safe = (gcchar*)(reinterpret_cast<uintptr_t>(&span_safe_bytes[0]));
+  span_gather<M, DeviceLds, THREADS, UNROLL>(g, m, pieces, safe, x0, len, a, lds, threadIdx.x);
+  __syncthreads();
+  span_write<M, DeviceLds, THREADS, UNROLL>(dst, len, a, lds, threadIdx.x);
+}
+
+template <int THREADS, int UNROLL>
+__global__ __launch_bounds__(THREADS) void mmr_span_kernel(const SpanGroup* __restrict__ groups, uint32_t n_groups,
+                                                           const SpanMember* __restrict__ members,
+                                                           const SpanPiece* __restrict__ pieces,
+                                                           const uint32_t* __restrict__ hints, uint32_t n,
+                                                           uint32_t xcd_group) {
+  __shared__ __attribute__((aligned(16))) uint8_t lds[kSpanLdsBytes];
+  const uint32_t ci = chunk_index(blockIdx.x, xcd_group);
+  if (ci >= n) return;  // uniform over the workgroup: no barrier is skipped by part of it
+  span_chunk<THREADS, UNROLL>(groups, n_groups, members, pieces, hints, ci, lds);
+}
+
+template <int THREADS, int UNROLL>
+__global__ __launch_bounds__(THREADS) void mmr_span_inline_kernel(const InlineSpanTable table, uint32_t xcd_group) {
+  __shared__ __attribute__((aligned(16))) uint8_t lds[kSpanLdsBytes];
+  const uint32_t ci = chunk_index(blockIdx.x, xcd_group);
+  if (ci >= table.n_chunks) return;
+  span_chunk<THREADS, UNROLL>(table.groups, table.n_groups, table.members, table.pieces, nullptr, ci, lds);
 }
 
 template <int THREADS, int UNROLL, bool NTL, bool NTS>
@@ -282,13 +368,53 @@ hipError_t launch_flat_copy(const void* src, void* dst, size_t bytes, hipStream_
   return hipGetLastError();
 }
 
-hipError_t launch_copy16(const mmr_copy_chunk* d_chunks, int64_t n, void* const* d_ptrs, uint32_t xcd_mode,
-                         hipStream_t stream) {
+hipError_t launch_copy_groups(const CopyGroup* d_groups, uint32_t n_groups, const CopyPiece* d_pieces,
+                              const uint32_t* d_hints, const uint32_t* starts, int64_t n, uint32_t xcd_mode,
+                              hipStream_t stream) {
   if (n == 0) return hipSuccess;
   if (hipError_t e = check_grid(n)) return e;
   const uint32_t group = xcd_group_of(n, xcd_mode);
-  hipLaunchKernelGGL((mmr_copy16_kernel<256, MMR_COPY16_UNROLL>), dim3(grid_size(n, group)), dim3(256), 0, stream, d_chunks,
-                     static_cast<uint32_t>(n), d_ptrs, group);
+  GroupStarts s;
+  for (uint32_t i = 0; i < kMaxDirectGroups; ++i) s.first[i] = starts && i < n_groups ? starts[i] : 0xffffffffu;
+  if (starts && n_groups <= kMaxDirectGroups)
+    hipLaunchKernelGGL((mmr_copy16_kernel<256, MMR_COPY16_UNROLL, true>), dim3(grid_size(n, group)), dim3(256), 0, stream,
+                       d_groups, n_groups, d_pieces, d_hints, static_cast<uint32_t>(n), group, s);
+  else
+    hipLaunchKernelGGL((mmr_copy16_kernel<256, MMR_COPY16_UNROLL, false>), dim3(grid_size(n, group)), dim3(256), 0, stream,
+                       d_groups, n_groups, d_pieces, d_hints, static_cast<uint32_t>(n), group, s);
+  return hipGetLastError();
+}
+
+hipError_t launch_copy_groups_inline(const InlineCopyTable& table, uint32_t xcd_mode, hipStream_t stream) {
+  const int64_t n = table.n_chunks;
+  if (n == 0) return hipSuccess;
+  if (hipError_t e = check_grid(n)) return e;
+  if (table.n_groups > kInlineCopyGroups) return hipErrorInvalidValue;
+  const uint32_t group = xcd_group_of(n, xcd_mode);
+  hipLaunchKernelGGL((mmr_copy16_inline_kernel<256, MMR_COPY16_UNROLL>), dim3(grid_size(n, group)), dim3(256), 0, stream,
+                     table, group);
+  return hipGetLastError();
+}
+
+hipError_t launch_spans(const SpanGroup* d_groups, uint32_t n_groups, const SpanMember* d_members,
+                        const SpanPiece* d_pieces, const uint32_t* d_hints, int64_t n, uint32_t xcd_mode,
+                        hipStream_t stream) {
+  if (n == 0) return hipSuccess;
+  if (hipError_t e = check_grid(n)) return e;
+  const uint32_t group = xcd_group_of(n, xcd_mode);
+  hipLaunchKernelGGL((mmr_span_kernel<256, MMR_SPAN_UNROLL>), dim3(grid_size(n, group)), dim3(256), 0, stream, d_groups,
+                     n_groups, d_members, d_pieces, d_hints, static_cast<uint32_t>(n), group);
+  return hipGetLastError();
+}
+
+hipError_t launch_spans_inline(const InlineSpanTable& table, uint32_t xcd_mode, hipStream_t stream) {
+  const int64_t n = table.n_chunks;
+  if (n == 0) return hipSuccess;
+  if (hipError_t e = check_grid(n)) return e;
+  if (table.n_groups > kInlineSpanGroups) return hipErrorInvalidValue;
+  const uint32_t group = xcd_group_of(n, xcd_mode);
+  hipLaunchKernelGGL((mmr_span_inline_kernel<256, MMR_SPAN_UNROLL>), dim3(grid_size(n, group)), dim3(256), 0, stream, table,
+                     group);
   return hipGetLastError();
 }
 

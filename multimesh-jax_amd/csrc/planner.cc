@@ -16,6 +16,8 @@
 
 #include <algorithm>
 #include <cstring>
+#include <map>
+#include <tuple>
 
 namespace mmr {
 namespace {
@@ -30,10 +32,45 @@ int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 constexpr int64_t kGenericMaxPairs = 768;  // (row, slot) pairs of one generic chunk
 
+// A box in canonical form: extent-1 dims dropped, dims in destination-major order, neighbours that are contiguous
+// on both sides merged, the run that is contiguous on both sides taken out as `w` bytes.
+struct CanonBox {
+  uint32_t src_slot, dst_slot;
+  int64_t so, dof;
+  std::vector<BoxDim> outer;
+  int64_t w;
+  bool fill;
+};
+
+// A group before the launch order is fixed.
+struct ProtoCopy {
+  CopyGroup g{};  // k, n1, n2, m1, m2, c1, d1, d2 set; the rest follows when the launch is assembled
+  std::vector<CopyPiece> pieces;
+  int array = 0;
+  uint32_t ordinal = 0;      // position among the groups of its (array, destination buffer)
+  uint64_t chunk_bytes = 0;  // destination bytes of one chunk of the widest piece
+};
+struct ProtoSpan {
+  SpanGroup g{};  // W, band_bytes, n1, span, head, div_W, div_n1 set
+  SpanMember m{};
+  std::vector<SpanPiece> pieces;
+  int array = 0;
+  uint32_t ordinal = 0;
+};
+
+constexpr size_t kSpanMaxPieces = 64;  // pieces of one destination row beyond which the span kernel's piece search costs too much
+
 class Builder {
  public:
-  Builder(mmr_plan* plan, uint32_t chunk_bytes, uint32_t generic_chunk_bytes, bool force_generic)
-      : plan_(plan), chunk_bytes_(chunk_bytes), generic_chunk_bytes_(generic_chunk_bytes), force_generic_(force_generic) {}
+  Builder(mmr_plan* plan, uint32_t chunk_bytes, uint32_t generic_chunk_bytes, uint32_t span_bytes, bool force_ragged,
+          bool no_span)
+      : plan_(plan), chunk_bytes_(chunk_bytes), generic_chunk_bytes_(generic_chunk_bytes), span_bytes_(span_bytes),
+        force_ragged_(force_ragged), no_span_(no_span) {}
+
+  std::vector<ProtoCopy> copies;
+  std::vector<ProtoSpan> spans;
+
+  void begin_array(int array) { array_ = array; }
 
   void add_box(uint32_t src_slot, uint32_t dst_slot, int64_t src_off, int64_t dst_off, const BoxDim* in, int rank,
                int itemsize) {
@@ -47,6 +84,7 @@ class Builder {
     const bool fill = src_slot == MMR_SLOT_FILL;
     if (fill) {
       plan_->stats.bytes_filled += volume * itemsize;
+      for (BoxDim& d : dims) d.s = d.d;  // a fill has no source side: let its dims merge by the destination alone
     } else {
       plan_->stats.bytes_moved += volume * itemsize;
       plan_->stats.n_boxes += 1;
@@ -71,12 +109,35 @@ class Builder {
       lower_transpose(src_slot, dst_slot, src_off, dst_off, dims, x, y, itemsize);
       return;
     }
-    int64_t w = itemsize;
+    CanonBox box{src_slot, dst_slot, fill ? 0 : src_off, dst_off, {}, itemsize, fill};
     if (run >= 0) {
-      w = dims[run].n * itemsize;
+      box.w = dims[run].n * itemsize;
       dims.erase(dims.begin() + run);
     }
-    lower_copy(src_slot, dst_slot, src_off, dst_off, dims, w, fill);
+    box.outer = std::move(dims);
+    tile_.push_back(std::move(box));
+  }
+
+  // All boxes of one destination tile are in: lower them.  A tile whose boxes are all 16-byte aligned becomes copy
+  // groups; otherwise the whole tile goes to the span kernel (every byte of a destination row must come through the
+  // same workgroup for it to leave as whole lines), and what that kernel does not take becomes generic chunks.
+  void finish_tile() {
+    bool aligned = !force_ragged_;
+    for (const CanonBox& b : tile_) {
+      uint64_t bits = static_cast<uint64_t>(b.so | b.dof | b.w);
+      for (const BoxDim& d : b.outer) bits |= static_cast<uint64_t>(d.s | d.d);
+      aligned &= (bits & 15u) == 0;
+    }
+    if (aligned) {
+      lower_copy_groups();
+    } else {
+      std::vector<CanonBox> rest;
+      if (no_span_) rest = tile_;
+      else lower_span_groups(&rest);
+      for (CanonBox& b : rest) lower_generic(b.src_slot, b.dst_slot, b.so, b.dof, b.outer, b.w, b.fill);
+    }
+    tile_.clear();
+    ordinal_ = 0;
   }
 
  private:
@@ -93,29 +154,335 @@ class Builder {
     return best;
   }
 
-  // Calls fn(src_delta, dst_delta) for every index combination of `dims`.
+  // Calls fn(index vector) for every index combination of `dims`.
   template <class Fn>
-  static void for_each_index(const std::vector<BoxDim>& dims, Fn&& fn) {
+  static void for_each_combo(const std::vector<BoxDim>& dims, Fn&& fn) {
     std::vector<int64_t> idx(dims.size(), 0);
-    int64_t so = 0, dof = 0;
     while (true) {
-      fn(so, dof);
+      fn(idx);
       int k = static_cast<int>(dims.size()) - 1;
       for (; k >= 0; --k) {
-        idx[k]++;
-        so += dims[k].s;
-        dof += dims[k].d;
-        if (idx[k] < dims[k].n) break;
-        so -= dims[k].s * dims[k].n;
-        dof -= dims[k].d * dims[k].n;
+        if (++idx[k] < dims[k].n) break;
         idx[k] = 0;
       }
       if (k < 0) break;
     }
   }
 
-  void emit_copy(uint32_t src_slot, uint32_t dst_slot, int64_t so, int64_t dof, int64_t w, int64_t n1, int64_t n2,
-                 int64_t s1, int64_t d1, int64_t s2, int64_t d2, bool fill) {
+  // Calls fn(src_delta, dst_delta) for every index combination of `dims`.
+  template <class Fn>
+  static void for_each_index(const std::vector<BoxDim>& dims, Fn&& fn) {
+    for_each_combo(dims, [&](const std::vector<int64_t>& idx) {
+      int64_t so = 0, dof = 0;
+      for (size_t i = 0; i < dims.size(); ++i) {
+        so += idx[i] * dims[i].s;
+        dof += idx[i] * dims[i].d;
+      }
+      fn(so, dof);
+    });
+  }
+
+  // Boxes that lie side by side in the same destination rows: equal row dims on the destination side and the same
+  // first row.  Returns index lists into tile_, each in ascending destination order.
+  std::vector<std::vector<int>> row_mates() const {
+    struct Key {
+      std::vector<int64_t> dims;  // (n, d) of every outer dim
+      int64_t origin;
+      bool operator<(const Key& o) const { return origin != o.origin ? origin < o.origin : dims < o.dims; }
+    };
+    std::map<Key, std::vector<int>> sets;
+    for (int i = 0; i < static_cast<int>(tile_.size()); ++i) {
+      const CanonBox& b = tile_[i];
+      Key key;
+      for (const BoxDim& d : b.outer) {
+        key.dims.push_back(d.n);
+        key.dims.push_back(d.d);
+      }
+      // the box is contiguous in the destination over its run and the dims that continue it (a chain of chain_bytes);
+      // its neighbours share the rows of the first dim above that chain
+      int64_t chain_bytes = b.w, pitch = 0;
+      for (int d = static_cast<int>(b.outer.size()) - 1; d >= 0; --d) {
+        if (b.outer[d].d != chain_bytes) {
+          pitch = b.outer[d].d;
+          break;
+        }
+        chain_bytes *= b.outer[d].n;
+      }
+      // a chain that does not fit between two rows has no neighbours in its rows
+      key.origin = pitch > 0 && b.dof % pitch + chain_bytes <= pitch ? b.dof - b.dof % pitch : b.dof;
+      sets[key].push_back(i);
+    }
+    std::vector<std::vector<int>> out;
+    for (auto& kv : sets) {
+      std::sort(kv.second.begin(), kv.second.end(), [&](int a, int b) { return tile_[a].dof < tile_[b].dof; });
+      out.push_back(std::move(kv.second));
+    }
+    std::sort(out.begin(), out.end(), [&](const std::vector<int>& a, const std::vector<int>& b) {
+      return tile_[a[0]].dof < tile_[b[0]].dof;
+    });
+    return out;
+  }
+
+  void lower_copy_groups() {
+    for (const std::vector<int>& mates : row_mates()) {
+      const CanonBox& first = tile_[mates[0]];
+      int64_t w_max = 0;
+      for (int i : mates) w_max = std::max(w_max, tile_[i].w);
+      const std::vector<BoxDim>& outer = first.outer;  // row structure; the mates share it on the destination side
+      const int64_t cb = chunk_bytes_;
+      // pieces: a box, or its column segments when its rows are longer than a chunk (near-equal segments on 256-byte
+      // boundaries of the row)
+      struct Seg {
+        int box;
+        int64_t c0, w;
+      };
+      std::vector<Seg> segs;
+      for (int i : mates) {
+        const int64_t w = tile_[i].w;
+        if (w > cb) {
+          const int64_t nseg = ceil_div(w, cb);
+          const int64_t seg = ceil_div(ceil_div(w, nseg), 256) * 256;
+          for (int64_t c0 = 0; c0 < w; c0 += seg) segs.push_back({i, c0, std::min(seg, w - c0)});
+        } else {
+          segs.push_back({i, 0, w});
+        }
+      }
+      int i1 = -1, i2 = -1;
+      int64_t m1 = 1, m2 = 1;
+      if (w_max > cb) {
+        i1 = pick_row_dim(outer, -1);  // one row per chunk
+        if (i1 >= 0) i2 = pick_row_dim(outer, i1);
+      } else {
+        const int64_t rows = std::max<int64_t>(1, cb / w_max);
+        i1 = pick_row_dim(outer, -1);
+        if (i1 >= 0) {
+          const BoxDim dim1 = outer[i1];
+          m1 = std::min(dim1.n, rows);
+          if (m1 < dim1.n && (dim1.d == w_max || dim1.s == w_max)) {
+            // Rows that abut on one side, cut into several chunks along this dim: keep the cuts on 128-byte lines of
+            // that side where a few rows less achieve it, so no line is shared by two workgroups (832-byte rows: 8 per
+            // chunk instead of 9 measured +3 %).
+            int64_t g = w_max, h = 128;
+            while (h != 0) {
+              const int64_t t = g % h;
+              g = h;
+              h = t;
+            }
+            const int64_t m = 128 / g;
+            if (m1 > m) m1 = m1 / m * m;
+          }
+          // Rows that continue the run on the destination side along one dim (A) and on the source side along
+          // another (B), as a fused layout permutation produces: take a 2-D block so both sides see runs of several
+          // rows instead of one side seeing single rows at a large stride.
+          int ia = -1, ib = -1;
+          if (!first.fill && outer.size() >= 2) {
+            for (int i = 0; i < static_cast<int>(outer.size()); ++i) {
+              if (outer[i].d == w_max && outer[i].s != w_max) ia = i;
+              if (outer[i].s == w_max && outer[i].d != w_max) ib = i;
+            }
+          }
+          if (ia >= 0 && ib >= 0 && rows >= 4) {
+            const BoxDim da = outer[ia], db = outer[ib];
+            int64_t na = 1;
+            while (na * 2 <= da.n && na * na * 4 <= rows) na *= 2;  // about sqrt(rows), a power of two
+            if (da.n * da.n <= 4 * rows) na = da.n;                  // or the whole of a short dim
+            i1 = ia;
+            m1 = std::min(na, da.n);
+            i2 = ib;
+            m2 = std::max<int64_t>(1, std::min(db.n, rows / m1));
+          } else {
+            i2 = pick_row_dim(outer, i1);
+            if (i2 >= 0) m2 = m1 == dim1.n ? std::max<int64_t>(1, std::min(outer[i2].n, rows / m1)) : 1;
+          }
+        }
+      }
+      const BoxDim dim1 = i1 >= 0 ? outer[i1] : BoxDim{1, 0, 0};
+      const BoxDim dim2 = i2 >= 0 ? outer[i2] : BoxDim{1, 0, 0};
+      // a third row dim rides along unblocked (the innermost of what is left); dims beyond it make groups of their own
+      int i3 = -1;
+      for (int i = static_cast<int>(outer.size()) - 1; i >= 0 && i3 < 0; --i)
+        if (i != i1 && i != i2) i3 = i;
+      const BoxDim dim3 = i3 >= 0 ? outer[i3] : BoxDim{1, 0, 0};
+      std::vector<BoxDim> rest;
+      std::vector<int> rest_index;
+      for (int i = 0; i < static_cast<int>(outer.size()); ++i)
+        if (i != i1 && i != i2 && i != i3) {
+          rest.push_back(outer[i]);
+          rest_index.push_back(i);
+        }
+      for_each_combo(rest, [&](const std::vector<int64_t>& idx) {
+        ProtoCopy pg;
+        pg.array = array_;
+        pg.ordinal = ordinal_++;
+        CopyGroup& g = pg.g;
+        g.k = static_cast<uint32_t>(segs.size());
+        g.n1 = static_cast<uint32_t>(dim1.n);
+        g.n2 = static_cast<uint32_t>(dim2.n);
+        g.n3 = static_cast<uint32_t>(dim3.n);
+        g.m1 = static_cast<uint32_t>(m1);
+        g.m2 = static_cast<uint32_t>(m2);
+        g.c1 = static_cast<uint32_t>(ceil_div(dim1.n, m1));
+        g.c12 = g.c1 * static_cast<uint32_t>(ceil_div(dim2.n, m2));
+        g.d1 = dim1.n > 1 ? dim1.d : 0;
+        g.d2 = dim2.n > 1 ? dim2.d : 0;
+        g.d3 = dim3.n > 1 ? dim3.d : 0;
+        pg.chunk_bytes = static_cast<uint64_t>(std::min(w_max, cb) * m1 * m2);
+        for (const Seg& sg : segs) {
+          const CanonBox& b = tile_[sg.box];
+          int64_t so = b.so + sg.c0, dof = b.dof + sg.c0;
+          for (size_t r = 0; r < rest.size(); ++r) {
+            so += idx[r] * b.outer[rest_index[r]].s;
+            dof += idx[r] * b.outer[rest_index[r]].d;
+          }
+          CopyPiece p{};
+          p.src_slot = b.src_slot;
+          p.dst_slot = b.dst_slot;
+          p.src = b.fill ? 0 : static_cast<uint64_t>(so);
+          p.dst = static_cast<uint64_t>(dof);
+          p.s1 = (i1 >= 0 && dim1.n > 1 && !b.fill) ? b.outer[i1].s : 0;
+          p.s2 = (i2 >= 0 && dim2.n > 1 && !b.fill) ? b.outer[i2].s : 0;
+          p.s3 = (i3 >= 0 && dim3.n > 1 && !b.fill) ? b.outer[i3].s : 0;
+          p.w = static_cast<uint32_t>(sg.w);
+          p.div_wv = make_fastdiv(std::max<uint32_t>(p.w >> 4, 1));
+          pg.pieces.push_back(p);
+        }
+        copies.push_back(std::move(pg));
+      });
+    }
+  }
+
+  // Ragged tile -> span groups.  Boxes the span kernel does not take are returned in *rest_out.
+  void lower_span_groups(std::vector<CanonBox>* rest_out) {
+    // Per box: the chain of dims over which it is contiguous in the destination (from the run outwards) and the head
+    // dims above it.  With head dims, the destination row is the innermost head dim's pitch and the chain dims are
+    // enumerated into pieces of that row (source-strided runs that abut in the destination); boxes with the same head
+    // and the same first row share the row.  Without head dims the box is dense by itself: its rows are the row.
+    struct Piece {
+      SpanPiece p;
+      std::vector<int64_t> row_s;  // source stride of every row dim of the band, innermost first
+    };
+    struct Band {
+      std::vector<BoxDim> rows;  // destination side, innermost first
+      int64_t W = 0, origin = 0;
+      uint32_t dst_slot = 0;
+      std::vector<Piece> pieces;
+      std::vector<int> boxes;
+      bool ok = true;
+    };
+    std::map<std::pair<int64_t, std::vector<int64_t>>, Band> bands;
+    for (int bi = 0; bi < static_cast<int>(tile_.size()); ++bi) {
+      const CanonBox& b = tile_[bi];
+      int64_t chain_bytes = b.w;
+      int head_n = static_cast<int>(b.outer.size());
+      while (head_n > 0 && b.outer[head_n - 1].d == chain_bytes) {
+        chain_bytes *= b.outer[head_n - 1].n;
+        --head_n;
+      }
+      std::vector<BoxDim> chain(b.outer.begin() + head_n, b.outer.end()), rows;
+      int64_t W, col;
+      if (head_n == 0) {  // dense by itself: rows of w bytes
+        W = b.w;
+        col = 0;
+        rows.assign(chain.rbegin(), chain.rend());
+        chain.clear();
+      } else {
+        W = b.outer[head_n - 1].d;
+        col = b.dof % W;
+        rows.assign(b.outer.rend() - head_n, b.outer.rend());
+      }
+      std::vector<int64_t> key_dims;
+      for (const BoxDim& d : rows) {
+        key_dims.push_back(d.n);
+        key_dims.push_back(d.d);
+      }
+      Band& band = bands[{b.dof - col, key_dims}];
+      if (band.boxes.empty()) {
+        band.rows = rows;
+        band.W = W;
+        band.origin = b.dof - col;
+        band.dst_slot = b.dst_slot;
+      }
+      band.boxes.push_back(bi);
+      size_t count = 1;
+      for (const BoxDim& d : chain) count *= static_cast<size_t>(d.n);
+      if (W > static_cast<int64_t>(kSpanMaxRowBytes) || band.pieces.size() + count > kSpanMaxPieces) {
+        band.ok = false;
+        continue;
+      }
+      for_each_index(chain, [&](int64_t ds, int64_t dd) {
+        Piece pc;
+        pc.p = SpanPiece{};
+        pc.p.src_slot = b.src_slot;
+        pc.p.src = b.fill ? 0 : static_cast<uint64_t>(b.so + ds);
+        pc.p.col = static_cast<uint32_t>(col + dd);
+        pc.p.w = static_cast<uint32_t>(b.w);
+        for (const BoxDim& d : rows) pc.row_s.push_back(b.fill ? 0 : d.s);
+        band.pieces.push_back(std::move(pc));
+      });
+    }
+    for (auto& kv : bands) {
+      Band& band = kv.second;
+      std::sort(band.pieces.begin(), band.pieces.end(), [](const Piece& a, const Piece& b) { return a.p.col < b.p.col; });
+      int64_t end = 0;
+      for (const Piece& pc : band.pieces) {  // the pieces must tile the row
+        band.ok &= pc.p.col == end;
+        end += pc.p.w;
+      }
+      band.ok &= end == band.W;
+      const BoxDim r1 = band.rows.empty() ? BoxDim{1, 0, 0} : band.rows[0];
+      band.ok &= band.rows.empty() || r1.d == band.W;  // rows abut
+      int64_t total_rows = 1;
+      for (const BoxDim& d : band.rows) total_rows *= d.n;
+      band.ok &= total_rows < (1ll << 31);
+      if (!band.ok) {
+        for (int bi : band.boxes) rest_out->push_back(tile_[bi]);
+        continue;
+      }
+      // n1 rows along the innermost dim; a second dim rides along when the rows stay dense across it; the dims above
+      // (and a second dim that is not dense) are enumerated, one band each
+      const bool dense2 = band.rows.size() > 1 && band.rows[1].d == r1.n * band.W;
+      const size_t skip = band.rows.empty() ? 0 : (dense2 ? 2 : 1);
+      const std::vector<BoxDim> rest(band.rows.begin() + skip, band.rows.end());
+      const int64_t n2 = dense2 ? band.rows[1].n : 1;
+      for_each_combo(rest, [&](const std::vector<int64_t>& idx) {
+        ProtoSpan ps;
+        ps.array = array_;
+        ps.ordinal = ordinal_++;
+        int64_t dst_shift = 0;
+        for (size_t r = 0; r < rest.size(); ++r) dst_shift += idx[r] * rest[r].d;
+        SpanGroup& g = ps.g;
+        g.W = static_cast<uint32_t>(band.W);
+        g.n1 = static_cast<uint32_t>(r1.n);
+        g.band_bytes = static_cast<uint64_t>(r1.n * n2 * band.W);
+        g.span = span_bytes_;
+        const uint64_t at = static_cast<uint64_t>(band.origin + dst_shift);
+        g.head = span_bytes_ - static_cast<uint32_t>(at % span_bytes_);
+        g.div_W = make_fastdiv(g.W);
+        g.div_n1 = make_fastdiv(g.n1);
+        ps.m.dst = at;
+        ps.m.dst_slot = band.dst_slot;
+        uint32_t wide = 0;
+        for (const Piece& pc : band.pieces) {
+          SpanPiece p = pc.p;
+          int64_t src_shift = 0;
+          for (size_t r = 0; r < rest.size(); ++r) src_shift += idx[r] * pc.row_s[skip + r];
+          p.src += static_cast<uint64_t>(src_shift);
+          p.s1 = pc.row_s.empty() ? 0 : pc.row_s[0];
+          p.s2 = dense2 ? pc.row_s[1] : 0;
+          p.wide_index = wide;
+          if (p.w >= 16) ++wide;
+          ps.pieces.push_back(p);
+        }
+        ps.m.k = static_cast<uint32_t>(ps.pieces.size());
+        ps.m.wide = wide;
+        ps.m.div_wide = make_fastdiv(std::max<uint32_t>(wide, 1));
+        spans.push_back(std::move(ps));
+      });
+    }
+  }
+
+  void emit_generic(uint32_t src_slot, uint32_t dst_slot, int64_t so, int64_t dof, int64_t w, int64_t n1, int64_t s1,
+                    int64_t d1, bool fill) {
     mmr_copy_chunk c{};
     c.src_slot = src_slot;
     c.dst_slot = dst_slot;
@@ -123,111 +490,48 @@ class Builder {
     c.dst_off = static_cast<uint64_t>(dof);
     c.w = static_cast<uint32_t>(w);
     c.n1 = static_cast<uint32_t>(n1);
-    c.n2 = static_cast<uint32_t>(n2);
+    c.n2 = 1;
     c.s1 = (n1 > 1 && !fill) ? s1 : 0;
     c.d1 = n1 > 1 ? d1 : 0;
-    c.s2 = (n2 > 1 && !fill) ? s2 : 0;
-    c.d2 = n2 > 1 ? d2 : 0;
-    uint64_t bits = c.src_off | c.dst_off | c.w | static_cast<uint64_t>(c.s1) | static_cast<uint64_t>(c.d1) |
-                    static_cast<uint64_t>(c.s2) | static_cast<uint64_t>(c.d2);
+    uint64_t bits = c.src_off | c.dst_off | c.w | static_cast<uint64_t>(c.s1) | static_cast<uint64_t>(c.d1);
     c.align = (bits & 15u) ? static_cast<uint32_t>(bits & (~bits + 1)) : 16u;
     if (fill) plan_->stats.n_fill_chunks += 1;
-    (c.align == 16 && !force_generic_ ? plan_->copy16 : plan_->generic).push_back(c);
+    plan_->generic.push_back(c);
   }
 
-  void lower_copy(uint32_t src_slot, uint32_t dst_slot, int64_t so, int64_t dof, std::vector<BoxDim>& outer, int64_t w,
-                  bool fill) {
-    // Rows that are not 16-byte aligned on both sides go to the generic kernel,
-    // which spends one lane per 16-byte slot plus ragged ends: give it half the
-    // bytes per workgroup so its workgroups live about as long as aligned ones.
-    uint64_t bits = static_cast<uint64_t>(so | dof | w);
-    for (const BoxDim& d : outer) bits |= static_cast<uint64_t>(d.s | d.d);
-    const bool aligned = (bits & 15u) == 0 && !force_generic_;
-    const int64_t cb = aligned ? chunk_bytes_ : generic_chunk_bytes_;
+  // Generic chunks: rows of one box along a single row dim, the other dims enumerated.
+  void lower_generic(uint32_t src_slot, uint32_t dst_slot, int64_t so, int64_t dof, const std::vector<BoxDim>& outer,
+                     int64_t w, bool fill) {
+    const int64_t cb = generic_chunk_bytes_;
     if (w > cb) {
       // long rows: split columns into near-equal segments on 256-byte boundaries of the row
       const int64_t nseg = ceil_div(w, cb);
       const int64_t seg = ceil_div(ceil_div(w, nseg), 256) * 256;
       for_each_index(outer, [&](int64_t ds, int64_t dd) {
         for (int64_t c0 = 0; c0 < w; c0 += seg)
-          emit_copy(src_slot, dst_slot, so + ds + c0, dof + dd + c0, std::min(seg, w - c0), 1, 1, 0, 0, 0, 0, fill);
+          emit_generic(src_slot, dst_slot, so + ds + c0, dof + dd + c0, std::min(seg, w - c0), 1, 0, 0, fill);
       });
       return;
     }
-    int64_t rows = std::max<int64_t>(1, cb / w);
-    if (!aligned) {
-      // The generic kernel spends one lane per (row, 16-byte slot) pair whatever the row holds: a chunk of very
-      // narrow rows sized by bytes alone (the one-byte pad column of a short edge tile: 5,632 rows) keeps its
-      // workgroup busy long after its neighbours have finished and becomes the tail of the launch.  Bound the
-      // pairs per chunk (3 per lane of a 256-lane workgroup) as well as the bytes.
-      const int64_t slots = (w + 15) / 16 + 1;
-      rows = std::max<int64_t>(1, std::min(rows, kGenericMaxPairs / slots));
-    }
-    int i1 = pick_row_dim(outer, -1);
+    // The generic kernel spends one lane per (row, 16-byte slot) pair whatever the row holds: a chunk of very narrow
+    // rows sized by bytes alone keeps its workgroup busy long after its neighbours have finished and becomes the tail
+    // of the launch.  Bound the pairs per chunk (3 per lane of a 256-lane workgroup) as well as the bytes.
+    const int64_t slots = (w + 15) / 16 + 1;
+    const int64_t rows = std::max<int64_t>(1, std::min(std::max<int64_t>(1, cb / w), kGenericMaxPairs / slots));
+    const int i1 = pick_row_dim(outer, -1);
     if (i1 < 0) {
-      emit_copy(src_slot, dst_slot, so, dof, w, 1, 1, 0, 0, 0, 0, fill);
+      emit_generic(src_slot, dst_slot, so, dof, w, 1, 0, 0, fill);
       return;
     }
-    BoxDim dim1 = outer[i1];
-    int64_t n1 = std::min(dim1.n, rows);
-    if (aligned && n1 < dim1.n && (dim1.d == w || dim1.s == w)) {
-      // Rows that abut on one side, cut into several chunks along this dim: keep the cuts on 128-byte lines of that
-      // side where a few rows less achieve it, so no line is shared by two workgroups (832-byte rows: 8 per chunk
-      // instead of 9 measured +3 %).
-      int64_t g = w, h = 128;
-      while (h != 0) {
-        const int64_t t = g % h;
-        g = h;
-        h = t;
-      }
-      const int64_t m = 128 / g;
-      if (n1 > m) n1 = n1 / m * m;
-    }
-    BoxDim dim2{1, 0, 0};
-    int64_t n2 = 1;
-    int i2 = -1;
-    // Rows that continue the run on the destination side along one dim (A) and on
-    // the source side along another (B), as a fused layout permutation produces:
-    // take a 2-D block so both sides see runs of several rows instead of one side
-    // seeing single rows at a large stride.
-    int ia = -1, ib = -1;
-    if (aligned && !fill && outer.size() >= 2) {
-      for (int i = 0; i < static_cast<int>(outer.size()); ++i) {
-        if (outer[i].d == w && outer[i].s != w) ia = i;
-        if (outer[i].s == w && outer[i].d != w) ib = i;
-      }
-    }
-    if (ia >= 0 && ib >= 0 && rows >= 4) {
-      const BoxDim da = outer[ia], db = outer[ib];
-      int64_t na = 1;
-      while (na * 2 <= da.n && na * na * 4 <= rows) na *= 2;  // about sqrt(rows), a power of two
-      if (da.n * da.n <= 4 * rows) na = da.n;                  // or the whole of a short dim
-      const int64_t nb = std::max<int64_t>(1, std::min(db.n, rows / na));
-      i1 = ia;
-      dim1 = da;
-      n1 = std::min(na, da.n);
-      i2 = ib;
-      dim2 = db;
-      n2 = nb;
-    } else if (aligned && n1 == dim1.n && rows / n1 >= 2) {  // the generic kernel walks a single row dimension
-      i2 = pick_row_dim(outer, i1);
-      if (i2 >= 0) {
-        dim2 = outer[i2];
-        n2 = std::min(dim2.n, rows / n1);
-      }
-    }
+    const BoxDim dim1 = outer[i1];
+    const int64_t n1 = std::min(dim1.n, rows);
     std::vector<BoxDim> rest;
     for (int i = 0; i < static_cast<int>(outer.size()); ++i)
-      if (i != i1 && i != i2) rest.push_back(outer[i]);
+      if (i != i1) rest.push_back(outer[i]);
     for_each_index(rest, [&](int64_t ds, int64_t dd) {
-      for (int64_t b2 = 0; b2 < dim2.n; b2 += n2) {
-        const int64_t m2 = std::min(n2, dim2.n - b2);
-        for (int64_t b1 = 0; b1 < dim1.n; b1 += n1) {
-          const int64_t m1 = std::min(n1, dim1.n - b1);
-          emit_copy(src_slot, dst_slot, so + ds + b2 * dim2.s + b1 * dim1.s, dof + dd + b2 * dim2.d + b1 * dim1.d, w, m1,
-                    m2, dim1.s, dim1.d, dim2.s, dim2.d, fill);
-        }
-      }
+      for (int64_t b1 = 0; b1 < dim1.n; b1 += n1)
+        emit_generic(src_slot, dst_slot, so + ds + b1 * dim1.s, dof + dd + b1 * dim1.d, w, std::min(n1, dim1.n - b1),
+                     dim1.s, dim1.d, fill);
     });
   }
 
@@ -292,7 +596,12 @@ class Builder {
   mmr_plan* plan_;
   uint32_t chunk_bytes_;
   uint32_t generic_chunk_bytes_;
-  bool force_generic_;
+  uint32_t span_bytes_;
+  bool force_ragged_;
+  bool no_span_;
+  int array_ = 0;
+  uint32_t ordinal_ = 0;
+  std::vector<CanonBox> tile_;
 };
 
 int plan_one_array(Builder& b, const Side& S, const Side& D, uint32_t slot_base) {
@@ -325,7 +634,10 @@ int plan_one_array(Builder& b, const Side& S, const Side& D, uint32_t slot_base)
         b.add_box(MMR_SLOT_FILL, dslot, 0, valid[i] * D.stride[i] * item, dims, rank, item);
       }
     }
-    if (empty) continue;
+    if (empty) {
+      b.finish_tile();
+      continue;
+    }
     int64_t t_lo[kMaxRank], t_n[kMaxRank], combos = 1;
     for (int i = 0; i < rank; ++i) {
       t_lo[i] = lo[i] / S.ext[i];
@@ -348,6 +660,7 @@ int plan_one_array(Builder& b, const Side& S, const Side& D, uint32_t slot_base)
       }
       b.add_box(slot_base + static_cast<uint32_t>(sdev), dslot, soff, doff, dims, rank, item);
     }
+    b.finish_tile();
   }
   return MMR_OK;
 }
@@ -366,18 +679,152 @@ std::string plan_key(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dst
   return k;
 }
 
+namespace {
+
+bool congruent(const ProtoCopy& a, const ProtoCopy& b) {
+  const CopyGroup &x = a.g, &y = b.g;
+  if (a.array != b.array || a.ordinal != b.ordinal || x.k != y.k || x.n1 != y.n1 || x.n2 != y.n2 || x.n3 != y.n3 ||
+      x.m1 != y.m1 || x.m2 != y.m2 || x.d1 != y.d1 || x.d2 != y.d2 || x.d3 != y.d3)
+    return false;
+  for (uint32_t j = 0; j < x.k; ++j)
+    if (a.pieces[j].w != b.pieces[j].w || a.pieces[j].dst != b.pieces[j].dst) return false;
+  return true;
+}
+
+bool congruent(const ProtoSpan& a, const ProtoSpan& b) {
+  const SpanGroup &x = a.g, &y = b.g;
+  return a.array == b.array && a.ordinal == b.ordinal && x.W == y.W && x.band_bytes == y.band_bytes && x.n1 == y.n1 &&
+         x.span == y.span && x.head == y.head;
+}
+
+// Fixes the launch order of the copy groups and lays them out in the plan.
+//   order 1: as generated; 2: by destination address; 3: by source address; 4: by destination, the tiles of an array
+//   interleaved in rounds of `fraction_bytes` per tile.
+void assemble_copies(std::vector<ProtoCopy>& protos, uint32_t order, int64_t fraction_bytes, mmr_plan* plan) {
+  std::vector<size_t> at(protos.size());
+  for (size_t i = 0; i < at.size(); ++i) at[i] = i;
+  auto dst_key = [&](size_t i) { return std::make_tuple(protos[i].pieces[0].dst_slot, protos[i].pieces[0].dst, i); };
+  if (order == 2) {
+    std::sort(at.begin(), at.end(), [&](size_t a, size_t b) { return dst_key(a) < dst_key(b); });
+  } else if (order == 3) {
+    std::sort(at.begin(), at.end(), [&](size_t a, size_t b) {
+      return std::make_tuple(protos[a].pieces[0].src_slot, protos[a].pieces[0].src, a) <
+             std::make_tuple(protos[b].pieces[0].src_slot, protos[b].pieces[0].src, b);
+    });
+  } else if (order == 4) {
+    std::sort(at.begin(), at.end(), [&](size_t a, size_t b) {
+      return std::make_tuple(protos[a].array, protos[a].ordinal, dst_key(a)) <
+             std::make_tuple(protos[b].array, protos[b].ordinal, dst_key(b));
+    });
+  }
+  uint32_t next_chunk = 0;
+  for (size_t i = 0; i < at.size();) {
+    const ProtoCopy& first = protos[at[i]];
+    size_t j = i + 1;
+    if (order == 4)
+      while (j < at.size() && congruent(first, protos[at[j]])) ++j;
+    CopyGroup g = first.g;
+    const uint32_t members = static_cast<uint32_t>(j - i);
+    const uint32_t member_chunks = g.k * g.c12 * g.n3;
+    // a round holds whole row blocks of all k pieces
+    uint32_t fraction = member_chunks;
+    if (members > 1) {
+      const uint64_t per = std::max<uint64_t>(first.chunk_bytes, 1);
+      fraction = static_cast<uint32_t>(std::max<uint64_t>(1, static_cast<uint64_t>(fraction_bytes) / per / g.k)) * g.k;
+    }
+    g.first_chunk = next_chunk;
+    g.n_chunks = members * member_chunks;
+    g.first_piece = static_cast<uint32_t>(plan->copy_pieces.size());
+    g.div_k = make_fastdiv(g.k);
+    g.div_c1 = make_fastdiv(g.c1);
+    g.div_c12 = make_fastdiv(g.c12);
+    g.div_m1 = make_fastdiv(g.m1);
+    g.div_last1 = make_fastdiv(g.n1 % g.m1 ? g.n1 % g.m1 : g.m1);
+    g.il = make_interleave(members, member_chunks, fraction);
+    // the lean chunk code: one pass, offsets inside a chunk in 32 bits (24 bits per factor for the fast multiplies)
+    uint64_t reach = 0, widest = 0, stride_bits = static_cast<uint64_t>(g.d1 | g.d2);
+    for (size_t m = i; m < j; ++m)
+      for (const CopyPiece& pc : protos[at[m]].pieces) {
+        widest = std::max<uint64_t>(widest, pc.w);
+        stride_bits |= static_cast<uint64_t>(pc.s1 | pc.s2);
+        reach = std::max<uint64_t>(reach, static_cast<uint64_t>(g.m2 - 1) * static_cast<uint64_t>(std::max(pc.s2, g.d2)) +
+                                              static_cast<uint64_t>(g.m1 - 1) * static_cast<uint64_t>(std::max(pc.s1, g.d1)) + pc.w);
+      }
+    g.lean = 0;
+    if (static_cast<uint64_t>(g.m1) * g.m2 * (widest >> 4) <= kLeanVectors && reach < (1ull << 32) && g.d1 >= 0 && g.d2 >= 0)
+      g.lean = stride_bits < (1ull << 24) ? 2 : 1;
+    for (size_t m = i; m < j; ++m)
+      for (const CopyPiece& pc : protos[at[m]].pieces) {
+        if (pc.src_slot == MMR_SLOT_FILL) plan->stats.n_fill_chunks += member_chunks / g.k;
+        plan->copy_pieces.push_back(pc);
+      }
+    plan->copy_groups.push_back(g);
+    next_chunk += g.n_chunks;
+    i = j;
+  }
+  plan->n_copy_chunks = next_chunk;
+}
+
+void assemble_spans(std::vector<ProtoSpan>& protos, uint32_t order, int64_t fraction_bytes, mmr_plan* plan) {
+  std::vector<size_t> at(protos.size());
+  for (size_t i = 0; i < at.size(); ++i) at[i] = i;
+  auto dst_key = [&](size_t i) { return std::make_tuple(protos[i].m.dst_slot, protos[i].m.dst, i); };
+  if (order == 2 || order == 3) {
+    std::sort(at.begin(), at.end(), [&](size_t a, size_t b) { return dst_key(a) < dst_key(b); });
+  } else if (order == 4) {
+    std::sort(at.begin(), at.end(), [&](size_t a, size_t b) {
+      return std::make_tuple(protos[a].array, protos[a].ordinal, dst_key(a)) <
+             std::make_tuple(protos[b].array, protos[b].ordinal, dst_key(b));
+    });
+  }
+  uint32_t next_chunk = 0;
+  for (size_t i = 0; i < at.size();) {
+    const ProtoSpan& first = protos[at[i]];
+    size_t j = i + 1;
+    if (order == 4)
+      while (j < at.size() && congruent(first, protos[at[j]])) ++j;
+    SpanGroup g = first.g;
+    const uint32_t members = static_cast<uint32_t>(j - i);
+    const uint32_t member_chunks = span_chunks(g.band_bytes, g.head, g.span);
+    const uint32_t fraction =
+        members > 1 ? static_cast<uint32_t>(std::max<int64_t>(1, fraction_bytes / g.span)) : member_chunks;
+    g.first_chunk = next_chunk;
+    g.n_chunks = members * member_chunks;
+    g.first_member = static_cast<uint32_t>(plan->span_members.size());
+    g.il = make_interleave(members, member_chunks, fraction);
+    for (size_t m = i; m < j; ++m) {
+      SpanMember mem = protos[at[m]].m;
+      mem.first_piece = static_cast<uint32_t>(plan->span_pieces.size());
+      plan->span_pieces.insert(plan->span_pieces.end(), protos[at[m]].pieces.begin(), protos[at[m]].pieces.end());
+      plan->span_members.push_back(mem);
+    }
+    plan->span_groups.push_back(g);
+    next_chunk += g.n_chunks;
+    i = j;
+  }
+  plan->n_span_chunks = next_chunk;
+}
+
+}  // namespace
+
+mmr_copy_chunk decoded_copy_chunk(const mmr_plan& plan, uint32_t ci) {
+  const uint32_t gi = find_group(plan.copy_groups.data(), static_cast<uint32_t>(plan.copy_groups.size()), nullptr, ci);
+  const CopyGroup& g = plan.copy_groups[gi];
+  const DecodedCopy d = decode_copy(g, ci - g.first_chunk);
+  return copy_chunk_of(g, plan.copy_pieces[d.piece], d);
+}
+
 int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int n, const mmr_plan_options& options,
                mmr_plan* plan) {
   if (n < 0 || (n > 0 && (!srcs || !dsts))) return fail(MMR_INVALID_ARGUMENT, "bad descriptor arrays");
   uint32_t chunk_bytes = options.chunk_bytes ? options.chunk_bytes : kDefaultChunkBytes;
   chunk_bytes = std::min<uint32_t>(std::max<uint32_t>(chunk_bytes, 256), 16u << 20) & ~255u;
   plan->options = options;
-  // Ragged rows cost more instructions per byte, so their chunks are half the aligned size when a size is asked
-  // for.  By default 7 KiB (8 rows of configuration 5's 820-byte rows), measured best on large arrays (360 MB of
-  // them: 5.13 TB/s against 5.00 at 5.5 KiB); a plan under ~58 MB gets proportionally smaller chunks, so that it
-  // still has some 8,000 of them to spread over 256 CUs (configuration 5, 45 MB, buffers not in the Infinity Cache:
-  // 4.35 TB/s at 5 KiB against 4.23 at 7 KiB and 3.95 at 8 KiB).
+  // Generic chunks (ragged boxes the span kernel does not take) cost more instructions per byte: half the aligned
+  // size when a size is asked for, 7 KiB by default, less for small plans so that they still make some 8,000 chunks.
   uint32_t generic_chunk_bytes = std::max<uint32_t>(chunk_bytes / 2, 256);
+  // Span of destination bytes per workgroup of the span kernel: the chunk size asked for, rounded to 128-byte lines.
+  uint32_t span_bytes = std::min<uint32_t>(std::max<uint32_t>(chunk_bytes & ~127u, 128), kSpanMaxBytes);
   if (options.chunk_bytes == 0) {
     int64_t payload = 0;
     for (int a = 0; a < n; ++a) {
@@ -386,13 +833,10 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
       payload += bytes;
     }
     generic_chunk_bytes = static_cast<uint32_t>(std::min<int64_t>(std::max<int64_t>(payload / 8192, 2048), 7168)) & ~255u;
+    span_bytes = kDefaultSpanBytes;
   }
-  Builder builder(plan, chunk_bytes, generic_chunk_bytes, (options.flags & MMR_PLAN_ALL_GENERIC) != 0);
-  struct SlotInfo {
-    int array;
-    int64_t shard_bytes;
-  };
-  std::vector<SlotInfo> slot_info;  // by slot
+  Builder builder(plan, chunk_bytes, generic_chunk_bytes, span_bytes, (options.flags & MMR_PLAN_ALL_GENERIC) != 0,
+                  (options.flags & MMR_PLAN_NO_SPAN) != 0);
   for (int a = 0; a < n; ++a) {
     Side S, D;
     if (int rc = make_side(srcs[a], &S)) return rc;
@@ -410,89 +854,29 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
     plan->srcs.push_back(srcs[a]);
     plan->dsts.push_back(dsts[a]);
     plan->slot_bases.push_back(plan->n_slots);
-    for (int64_t k = 0; k < S.dev_count; ++k) slot_info.push_back({a, S.shard_bytes});
-    for (int64_t k = 0; k < D.dev_count; ++k) slot_info.push_back({a, D.shard_bytes});
+    builder.begin_array(a);
     if (int rc = plan_one_array(builder, S, D, static_cast<uint32_t>(plan->n_slots))) return rc;
     plan->n_slots += S.dev_count + D.dev_count;
   }
-  // A plan that is mostly ragged rows: its few aligned chunks ride along in the
-  // generic table (the generic kernel handles aligned rows too), one launch less.
-  if (!plan->generic.empty() && !plan->copy16.empty()) {
-    int64_t aligned_bytes = 0, generic_bytes = 0;
-    bool one_dim = true;
-    for (const mmr_copy_chunk& c : plan->copy16) {
-      aligned_bytes += static_cast<int64_t>(c.w) * c.n1 * c.n2;
-      one_dim &= c.n2 == 1;
-    }
-    for (const mmr_copy_chunk& c : plan->generic) generic_bytes += static_cast<int64_t>(c.w) * c.n1 * c.n2;
-    if (one_dim && aligned_bytes * 4 < generic_bytes) {
-      plan->generic.insert(plan->generic.end(), plan->copy16.begin(), plan->copy16.end());
-      plan->copy16.clear();
-    }
-  }
-  // Default order: aligned chunks and transpose tiles by destination address; ragged (generic) chunks by
-  // destination with the tiles of an array interleaved (4), measured +12 % on configuration 5.
+  // Launch order.  Copy groups: by destination address unless the options say otherwise.  Span groups (ragged rows):
+  // by destination with the tiles of an array interleaved - chunks of neighbouring tiles that cover the same rows
+  // read the same source lines at the edges of their column ranges, and runs of table neighbours share an XCD's L2.
+  const int64_t fraction_kib = (options.flags >> 8) & 0xffffu;
+  const uint32_t copy_order = options.order ? options.order : 2;
+  const uint32_t span_order = options.order ? options.order : 4;
+  assemble_copies(builder.copies, copy_order, (fraction_kib ? fraction_kib : 64) * 1024, plan);
+  assemble_spans(builder.spans, span_order, (fraction_kib ? fraction_kib : kDefaultSpanFractionKib) * 1024, plan);
+  if (plan->n_copy_chunks > 0x7ff00000u || plan->n_span_chunks > 0x7ff00000u)
+    return fail(MMR_INVALID_ARGUMENT, "plan of more than 2^31 chunks");
   const uint32_t order = options.order ? options.order : 2;
-  const uint32_t generic_order = options.order ? options.order : 4;
-  if (order == 2 || order == 3) {
-    // Sorting 72-byte records directly dominated the planning time of large batches: sort (key, index) triples
-    // and permute once.  The index as last key keeps equal keys (fill chunks share FILL as source) in emission order.
-    auto sort_copy = [order](std::vector<mmr_copy_chunk>& table) {
-      struct Key {
-        uint64_t slot, off;
-        uint32_t index;
-      };
-      std::vector<Key> keys(table.size());
-      bool sorted = true;
-      for (size_t i = 0; i < table.size(); ++i) {
-        const mmr_copy_chunk& c = table[i];
-        keys[i] = order == 2 ? Key{c.dst_slot, c.dst_off, static_cast<uint32_t>(i)}
-                             : Key{c.src_slot, c.src_off, static_cast<uint32_t>(i)};
-        if (i > 0 && std::tie(keys[i].slot, keys[i].off) < std::tie(keys[i - 1].slot, keys[i - 1].off)) sorted = false;
-      }
-      if (sorted) return;
-      std::sort(keys.begin(), keys.end(), [](const Key& a, const Key& b) {
-        return std::tie(a.slot, a.off, a.index) < std::tie(b.slot, b.off, b.index);
-      });
-      std::vector<mmr_copy_chunk> out(table.size());
-      for (size_t i = 0; i < keys.size(); ++i) out[i] = table[keys[i].index];
-      table.swap(out);
-    };
-    sort_copy(plan->copy16);
-    if (generic_order == order) sort_copy(plan->generic);
-  }
-  if (order == 4 || generic_order == 4) {
-    // Ragged rows: chunks of different destination tiles that cover the same rows read the same source lines at
-    // the edges of their column ranges.  Cut every destination buffer into equal fractions and keep the chunks of
-    // one fraction of all tiles of an array together (inside a fraction: by destination address), so that they
-    // run at the same time on the same XCD and the shared lines are fetched once.
-    const int64_t fraction_kib = (options.flags >> 8) & 0xffffu;  // tuning knob; 0 = default
-    const int64_t fraction_bytes = (fraction_kib ? fraction_kib : 64) * 1024;
-    auto sort_interleaved = [&](std::vector<mmr_copy_chunk>& table) {
-      struct Key {
-        uint64_t array, fraction, slot, off;
-        uint32_t index;
-      };
-      std::vector<Key> keys(table.size());
-      for (size_t i = 0; i < table.size(); ++i) {
-        const mmr_copy_chunk& c = table[i];
-        const SlotInfo& info = slot_info[c.dst_slot];
-        const uint64_t fractions = std::max<int64_t>(1, info.shard_bytes / fraction_bytes);
-        keys[i] = Key{static_cast<uint64_t>(info.array),
-                      info.shard_bytes > 0 ? c.dst_off * fractions / static_cast<uint64_t>(info.shard_bytes) : 0, c.dst_slot,
-                      c.dst_off, static_cast<uint32_t>(i)};
-      }
-      std::sort(keys.begin(), keys.end(), [](const Key& a, const Key& b) {
-        return std::tie(a.array, a.fraction, a.slot, a.off, a.index) < std::tie(b.array, b.fraction, b.slot, b.off, b.index);
-      });
-      std::vector<mmr_copy_chunk> out(table.size());
-      for (size_t i = 0; i < keys.size(); ++i) out[i] = table[keys[i].index];
-      table.swap(out);
-    };
-    if (order == 4) sort_interleaved(plan->copy16);
-    sort_interleaved(plan->generic);
-  }
   if (order == 2 || order == 3 || order == 4) {
+    auto sort_generic = [order](std::vector<mmr_copy_chunk>& table) {
+      std::stable_sort(table.begin(), table.end(), [order](const mmr_copy_chunk& a, const mmr_copy_chunk& b) {
+        return order == 3 ? std::tie(a.src_slot, a.src_off) < std::tie(b.src_slot, b.src_off)
+                          : std::tie(a.dst_slot, a.dst_off) < std::tie(b.dst_slot, b.dst_off);
+      });
+    };
+    sort_generic(plan->generic);
     // Tiles: by destination in blocks of 8 x 8 tiles rather than row after row, so the workgroups in flight
     // together cover a compact region with long contiguous pieces on the source side as well as on the
     // destination side (measured +10 % over plain destination order).
@@ -517,15 +901,22 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
                      return std::make_pair(a.itemsize, !transpose_is_vector(a)) < std::make_pair(b.itemsize, !transpose_is_vector(b));
                    });
   plan->stats.order_used = options.order;
-  plan->stats.interleave_kib = options.order == 4 ? (((options.flags >> 8) & 0xffffu) ? ((options.flags >> 8) & 0xffffu) : 64) : 0;
+  plan->stats.interleave_kib = options.order == 4 ? (fraction_kib ? fraction_kib : 64) : 0;
   plan->stats.n_arrays = n;
-  plan->stats.n_copy16_chunks = static_cast<int64_t>(plan->copy16.size());
+  plan->stats.n_copy16_chunks = plan->n_copy_chunks;
+  plan->stats.n_span_chunks = plan->n_span_chunks;
   plan->stats.n_copy_generic_chunks = static_cast<int64_t>(plan->generic.size());
   plan->stats.n_transpose_chunks = static_cast<int64_t>(plan->transposes.size());
+  plan->stats.n_groups = static_cast<int64_t>(plan->copy_groups.size() + plan->span_groups.size());
+  plan->stats.n_pieces = static_cast<int64_t>(plan->copy_pieces.size() + plan->span_pieces.size());
   plan->stats.n_slots = plan->n_slots;
-  plan->stats.table_bytes =
-      static_cast<int64_t>((plan->copy16.size() + plan->generic.size()) * sizeof(mmr_copy_chunk) +
-                           plan->transposes.size() * sizeof(mmr_transpose_chunk) + plan->n_slots * sizeof(void*));
+  plan->stats.table_bytes = static_cast<int64_t>(
+      plan->copy_groups.size() * sizeof(CopyGroup) + plan->copy_pieces.size() * sizeof(CopyPiece) +
+      plan->span_groups.size() * sizeof(SpanGroup) + plan->span_members.size() * sizeof(SpanMember) +
+      plan->span_pieces.size() * sizeof(SpanPiece) +
+      (((plan->n_copy_chunks + 63) >> 6) + ((plan->n_span_chunks + 63) >> 6)) * sizeof(uint32_t) +
+      plan->generic.size() * sizeof(mmr_copy_chunk) + plan->transposes.size() * sizeof(mmr_transpose_chunk) +
+      ((plan->generic.empty() && plan->transposes.empty()) ? 0 : plan->n_slots * sizeof(void*)));
   return MMR_OK;
 }
 
@@ -559,7 +950,41 @@ int mmr_plan_get_stats(const mmr_plan* plan, mmr_plan_stats* out) {
 
 int64_t mmr_plan_get_copy_chunks(const mmr_plan* plan, int32_t kind, mmr_copy_chunk* out, int64_t capacity) {
   if (!plan) return 0;
-  const auto& v = kind == 0 ? plan->copy16 : plan->generic;
+  if (kind == 0) {  // decoded from the group table, in launch order
+    if (!out) return plan->n_copy_chunks;
+    const int64_t n = std::min<int64_t>(capacity, plan->n_copy_chunks);
+    for (int64_t i = 0; i < n; ++i) out[i] = mmr::decoded_copy_chunk(*plan, static_cast<uint32_t>(i));
+    return n;
+  }
+  if (kind == 2) {  // the row pieces of the span groups, one record each: n2 x n1 rows of w bytes
+    std::vector<mmr_copy_chunk> v;
+    for (const mmr::SpanGroup& g : plan->span_groups)
+      for (uint32_t t = 0; t < g.il.members; ++t) {
+        const mmr::SpanMember& m = plan->span_members[g.first_member + t];
+        for (uint32_t j = 0; j < m.k; ++j) {
+          const mmr::SpanPiece& p = plan->span_pieces[m.first_piece + j];
+          mmr_copy_chunk c{};
+          c.src_slot = p.src_slot;
+          c.dst_slot = m.dst_slot;
+          c.src_off = p.src;
+          c.dst_off = m.dst + p.col;
+          c.w = p.w;
+          c.n1 = g.n1;
+          c.n2 = static_cast<uint32_t>(g.band_bytes / g.W / g.n1);
+          c.align = 1;
+          c.s1 = p.s1;
+          c.d1 = g.W;
+          c.s2 = p.s2;
+          c.d2 = static_cast<int64_t>(g.W) * g.n1;
+          v.push_back(c);
+        }
+      }
+    if (!out) return static_cast<int64_t>(v.size());
+    const int64_t n = std::min<int64_t>(capacity, static_cast<int64_t>(v.size()));
+    if (n > 0) std::memcpy(out, v.data(), sizeof(mmr_copy_chunk) * n);
+    return n;
+  }
+  const auto& v = plan->generic;
   int64_t n = std::min<int64_t>(capacity, static_cast<int64_t>(v.size()));
   if (out && n > 0) std::memcpy(out, v.data(), sizeof(mmr_copy_chunk) * n);
   return out ? n : static_cast<int64_t>(v.size());

@@ -124,6 +124,26 @@ def config(index: int, scale: int = 1) -> List[dict]:
     raise ValueError("configuration %r" % (index,))
 
 
+def load_json(path: str) -> List[dict]:
+    """Arrays of a user-defined workload: a JSON list of dicts with the keys described at the top of this file."""
+    import json
+    with open(path) as f:
+        arrays = json.load(f)
+    for a in arrays:
+        a["shape"] = tuple(int(s) for s in a["shape"])
+        for side in ("src", "dst"):
+            a[side]["dims"] = [tuple(int(v) for v in d) for d in a[side]["dims"]]
+        a.setdefault("seed", 0)
+        a.setdefault("dist", "raw")
+    return arrays
+
+
+def side(shape: Sequence[int], sharding: Sequence[int], dev_start: int, replication: int = 1,
+         minor_to_major: Optional[Sequence[int]] = None) -> dict:
+    """One side of a workload array: row-major device order over `sharding` tiles per dim."""
+    return _side(shape, sharding, dev_start, replication, minor_to_major)
+
+
 def algorithmic_bytes(arrays: Sequence[dict]) -> int:
     """2 x valid elements x itemsize per array: each element read once from one
     source replica and written once per destination shard that owns it."""

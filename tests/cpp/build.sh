@@ -4,9 +4,9 @@
 set -euo pipefail
 here="$(cd "$(dirname "${BASH_SOURCE[0]}")" && pwd)"
 root="${here}/../.."
-g++ -O2 -std=c++20 -Wall -Wextra -I"${root}/include" -I"${root}/multimesh-jax_amd/csrc" \
-  "${here}/hip_execute_context_test.cc" \
-  -L"${root}/multimesh-jax_amd" -lmmreshard -L"${root}/oracle" -lreshard_oracle \
+g++ -O2 -std=c++20 -Wall -Wextra -Wno-unknown-pragmas -D__HIP_PLATFORM_AMD__ -I/opt/rocm/include -I"${root}/include" \
+  -I"${root}/multimesh-jax_amd/csrc" "${here}/hip_execute_context_test.cc" \
+  -L"${root}/multimesh-jax_amd" -lmmreshard -L"${root}/oracle" -lreshard_oracle -L/opt/rocm/lib -lamdhip64 \
   -Wl,-rpath,'$ORIGIN/../../multimesh-jax_amd' -Wl,-rpath,'$ORIGIN/../../oracle' -Wl,-rpath,/opt/rocm/lib \
   -o "${here}/hip_execute_context_test"
 echo "built ${here}/hip_execute_context_test"

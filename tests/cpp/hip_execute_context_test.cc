@@ -12,7 +12,10 @@
 #include <string>
 #include <vector>
 
+#include <hip/hip_runtime_api.h>
+
 #include "hip_execute_context.h"
+#include "shard_buffer.h"
 
 extern "C" {
 // oracle/reshard_cpu.c
@@ -133,23 +136,31 @@ static int run() {
   // a device outside the store's device list has no shard to slice
   EXPECT(throws([&] { ctx->SliceLocalShard(0, root[0]); }, "holds no shard"));
 
-  // a second execution over the same stores reuses plan and pointer table
-  for (int d = 0; d < kLocal; ++d) ctx->Reshard(d, d, param[d], root[d]);
-  EXPECT(ctx->Stats().reshard_calls == 2);
+  // later executions over the same stores reuse the plan; the second builds the device tables, the third finds them
+  for (int rep = 0; rep < 2; ++rep) {
+    for (int d = 0; d < kLocal; ++d) ctx->Reshard(d, d, param[d], root[d]);
+    ctx->Flush();
+  }
+  EXPECT(ctx->Stats().reshard_calls == 3);
   EXPECT(ctx->Stats().plans_built == 1);
+  EXPECT(ctx->Stats().inline_launches == 1);
+  EXPECT(ctx->Stats().bindings_built == 1);
   EXPECT(ctx->Stats().binding_cache_hits == 1);
 
-  // offload to pinned host memory and back, issued by every local device like any other op
+  // offload to the pinned host cache and back, issued by every local device like any other op; the host never waits
   {
-    const int64_t dev_bytes = ctx->Stats().bytes_allocated;
-    for (int d = 0; d < kLocal; ++d) ctx->OffloadDtoH(d, {root[d]}, {}, "task");
-    EXPECT(ctx->Stats().bytes_allocated < dev_bytes);
-    EXPECT(ctx->Stats().host_bytes_allocated > 0);
+    const mmr_context_stats before = ctx->Stats();
+    for (int d = 0; d < kLocal; ++d) ctx->OffloadDtoH(d, {root[d]}, {param[d]}, "task");
+    EXPECT(ctx->Stats().host_bytes_allocated > before.host_bytes_allocated);
     // the mock's invariant: an offloaded store cannot take part in device work
     EXPECT(throws([&] { ctx->Reshard(0, 0, param[0], root[0]); }, "offloaded"));  // consumes no position
     for (int d = 0; d < kLocal; ++d) ctx->OffloadHtoD(d, {root[d]}, "task");
-    EXPECT(ctx->Stats().bytes_allocated == dev_bytes);
-    EXPECT(ctx->Stats().host_bytes_allocated == 0);
+    EXPECT(ctx->Stats().host_blocking_syncs == before.host_blocking_syncs);
+    EXPECT(ctx->Stats().device_allocations == before.device_allocations);  // the tile came back out of the device cache
+    for (int d = 0; d < kLocal; ++d) ctx->OffloadDtoH(d, {root[d]}, {}, "task");  // pinned buffer from the host cache
+    for (int d = 0; d < kLocal; ++d) ctx->OffloadHtoD(d, {root[d]}, "task");
+    EXPECT(ctx->Stats().host_cache_hits == before.host_cache_hits + 1);
+    EXPECT(ctx->Stats().host_bytes_allocated == before.host_bytes_allocated + 4 * ShardSize(dst));  // still one pinned buffer
     std::vector<uint16_t> got(expect[0].size());
     ctx->CopyShardToHost(root[8], got.data(), got.size() * 2);
     EXPECT(std::memcmp(got.data(), expect[0].data(), got.size() * 2) == 0);
@@ -300,6 +311,19 @@ static int run() {
       else EXPECT(roots[0][0].unique_id != first_root);
       EXPECT(sc->Stats().stores_live == stores_before + 1 + 2);  // t0 + this run's two roots (last run's are gone)
     }
+    // Steady state of a training loop: fresh ROOT stores every execution, yet no allocation, no table upload and no
+    // wait on the device from the third execution on (the roots' memory comes back through the allocator's pool at
+    // the same addresses, so the device tables bound to them are found again).
+    for (int warm = 0; warm < 2; ++warm) schedule.Execute(*sc, params);
+    const mmr_context_stats steady0 = sc->Stats();
+    for (int step = 0; step < 5; ++step) schedule.Execute(*sc, params);
+    const mmr_context_stats steady1 = sc->Stats();
+    EXPECT(steady1.reshard_calls - steady0.reshard_calls == 10);
+    EXPECT(steady1.device_allocations == steady0.device_allocations);
+    EXPECT(steady1.bindings_built == steady0.bindings_built);
+    EXPECT(steady1.plans_built == steady0.plans_built);
+    EXPECT(steady1.host_blocking_syncs == steady0.host_blocking_syncs);
+    EXPECT(steady1.pool_hits - steady0.pool_hits == 10);
   }
 
   // Free(keep_in_cache) + CreateStore(allocate_from_cache) on a fresh context
@@ -325,6 +349,126 @@ static int run() {
   EXPECT(h4.unique_id == h5.unique_id);
   ctx2->Destroy(h2);
   ctx2->Destroy(h3);
+  // Free without keep_in_cache only drops the copy it is given (zuku_execute_context_impl.cc:513-514): every other
+  // copy of the handle still works, and the store lives until the last one goes
+  {
+    StoreHandle k0 = ctx2->CreateStore(0, 0, small), k1 = ctx2->CreateStore(1, 1, small);
+    const int64_t live = ctx2->Stats().stores_live;
+    ctx2->Free(0, k0, /*keep_in_cache=*/false);
+    EXPECT(ctx2->Stats().stores_live == live);
+    EXPECT(ctx2->SliceLocalShard(0, k0) != nullptr);
+    ctx2->Destroy(k0);
+    ctx2->Destroy(k1);
+    EXPECT(ctx2->Stats().stores_live == live - 1);
+  }
+  // CreateStoreConfig::min_cache_size: the cache of the descriptor is filled to that many buffers at once
+  {
+    ShardedShape other{SupportedType::F32, {{{6000, 2, 0}}, DeviceList::Create(0, 2)}, {}};  // a size nothing has freed yet
+    const mmr_context_stats b = ctx2->Stats();
+    StoreHandle m0 = ctx2->CreateStore(0, 0, other, {.allocate_from_cache = true, .min_cache_size = 3});
+    StoreHandle m1 = ctx2->CreateStore(1, 1, other, {.allocate_from_cache = true, .min_cache_size = 3});
+    EXPECT(ctx2->Stats().device_allocations == b.device_allocations + 3);
+    StoreHandle n0 = ctx2->CreateStore(0, 0, other, {.allocate_from_cache = true});
+    StoreHandle n1 = ctx2->CreateStore(1, 1, other, {.allocate_from_cache = true});
+    StoreHandle o0 = ctx2->CreateStore(0, 0, other, {.allocate_from_cache = true});
+    StoreHandle o1 = ctx2->CreateStore(1, 1, other, {.allocate_from_cache = true});
+    EXPECT(ctx2->Stats().device_allocations == b.device_allocations + 3);
+    EXPECT(ctx2->Stats().cache_hits == b.cache_hits + 2);
+    EXPECT(m0.unique_id == m1.unique_id && n0.unique_id != m0.unique_id && o1.unique_id != n1.unique_id);
+  }
+
+  // The buffer wrapper (MultiMeshPjRtBuffer): native shards -> store, store -> zero-copy view that pins the store.
+  {
+    auto bc = HipExecuteContext::Create(local);
+    hipStream_t producer = nullptr;
+    EXPECT(hipStreamCreateWithFlags(&producer, hipStreamNonBlocking) == hipSuccess);
+    auto producer_stream = std::make_shared<MultiMeshStream>(producer);
+    // native shards in device memory, written by work on the producer's stream that nobody waits for on the host
+    std::vector<void*> device_shards(8, nullptr);
+    std::vector<std::unique_ptr<ShardBuffer>> natives(kLocal);
+    for (int d = 0; d < 8; ++d) {
+      EXPECT(hipMalloc(&device_shards[d], shards[d].size() * 2) == hipSuccess);
+      EXPECT(hipMemcpyAsync(device_shards[d], shards[d].data(), shards[d].size() * 2, hipMemcpyHostToDevice, producer) ==
+             hipSuccess);
+    }
+    const mmr_context_stats b0 = bc->Stats();
+    std::vector<StoreHandle> as_store(kLocal);
+    for (int d = 0; d < kLocal; ++d) {
+      auto native = std::make_shared<NativeBuffer>(d < 8 ? device_shards[d] : nullptr, d < 8 ? shards[d].size() * 2 : 0);
+      natives[d] = std::make_unique<ShardBuffer>(native, std::vector<int64_t>{4, 64, 256}, std::vector<int64_t>{4, 64, 32},
+                                                 SupportedType::BF16, bc, d, d, "param");
+      EXPECT(natives[d]->has_native_buffer() && natives[d]->HasValidShard());
+      as_store[d] = natives[d]->ToStore(src, producer_stream);
+    }
+    EXPECT(bc->Stats().host_blocking_syncs == b0.host_blocking_syncs);  // ordered by an event, not by the host
+    // output buffers backed by a store, as Execute hands them out (mm_pjrt_executable.cc:684-689)
+    std::vector<std::unique_ptr<ShardBuffer>> outs(kLocal);
+    {
+      std::vector<StoreHandle> r(kLocal);
+      for (int d = 0; d < kLocal; ++d) r[d] = bc->CreateStore(d, d, dst, {.name = "out"});
+      for (int d = 0; d < kLocal; ++d) bc->Reshard(d, d, as_store[d], r[d]);
+      for (int d = 0; d < kLocal; ++d)
+        outs[d] = std::make_unique<ShardBuffer>(r[d], std::vector<int64_t>{4, 64, 256}, std::vector<int64_t>{4, 16, 256},
+                                                SupportedType::BF16, bc, d, d, "out");
+    }  // the executable's own handles are gone: the buffers hold the store now
+    for (int d = 0; d < kLocal; ++d) {
+      EXPECT(outs[d]->has_store());
+      EXPECT(outs[d]->HasValidShard() == (d >= 8));
+      EXPECT(outs[d]->GetOnDeviceSizeInBytes() == static_cast<size_t>(ShardSize(dst)));
+      EXPECT(outs[d]->ToStore(dst, producer_stream).unique_id == outs[d]->store().unique_id);  // already a store
+    }
+    // a view of device 9's tile, then every buffer and handle of the store goes
+    std::unique_ptr<ShardBuffer> view = outs[9]->SliceLocalShard();
+    EXPECT(view->has_native_buffer() && view->name() == "out.sliced");
+    ShardBuffer::ExternalReference ext = outs[10]->AcquireExternalReference();
+    EXPECT(ext.data != nullptr && ext.store.has_value());
+    const int64_t live_before = bc->Stats().stores_live;
+    outs.clear();
+    EXPECT(bc->Stats().stores_live == live_before);  // the view and the external reference pin it
+    // other work reuses freed memory if it can: a reshard into a new store of the same descriptor
+    {
+      std::vector<StoreHandle> r2(kLocal);
+      for (int d = 0; d < kLocal; ++d) r2[d] = bc->CreateStore(d, d, dst);
+      std::vector<std::vector<uint16_t>> other(8, std::vector<uint16_t>(4 * 64 * 32, 0x5A5A));
+      std::vector<StoreHandle> p2(kLocal);
+      for (int d = 0; d < kLocal; ++d)
+        p2[d] = bc->AssembleShards(d, d, src, Shard{d < 8 ? other[d].data() : nullptr, d, d < 8 ? other[d].size() * 2 : 0});
+      for (int d = 0; d < kLocal; ++d) bc->Reshard(d, d, p2[d], r2[d]);
+      bc->Flush();
+    }
+    std::vector<uint16_t> got(expect[1].size());
+    view->ToLiteral(got.data(), got.size() * 2);
+    EXPECT(std::memcmp(got.data(), expect[1].data(), got.size() * 2) == 0);  // device 9 = second destination tile
+    EXPECT(hipMemcpy(got.data(), ext.data, got.size() * 2, hipMemcpyDeviceToHost) == hipSuccess);
+    EXPECT(std::memcmp(got.data(), expect[2].data(), got.size() * 2) == 0);
+    view.reset();
+    ext = ShardBuffer::ExternalReference{};
+    EXPECT(bc->Stats().stores_live == live_before - 1);  // now it is gone
+    natives.clear();
+    as_store.clear();
+    bc.reset();
+    for (void* p : device_shards) EXPECT(hipFree(p) == hipSuccess);
+    EXPECT(hipStreamDestroy(producer) == hipSuccess);
+  }
+
+  // Checking mode kept from the reference's mock: the same schedule hashes the same on every run, a different one does
+  // not; every reshard operand is checked for a tile on each of its devices.
+  {
+    auto run_schedule = [&](bool swap) -> int64_t {
+      auto hc = HipExecuteContext::Create({0, 1, 2, 3});
+      hc->SetCheckInvariants(true);
+      ShardedShape a{SupportedType::F32, {{{32, 2, 0}, {16, 1, 1}}, DeviceList::Create(0, 2)}, {}};
+      ShardedShape b{SupportedType::F32, {{{32, 1, 0}, {16, 2, 1}}, DeviceList::Create(2, 2)}, {}};
+      std::vector<StoreHandle> x(4), y(4);
+      for (int d = 0; d < 4; ++d) x[d] = hc->CreateStore(d, d, swap ? b : a);
+      for (int d = 0; d < 4; ++d) y[d] = hc->CreateStore(d, d, swap ? a : b);
+      for (int d = 0; d < 4; ++d) hc->Reshard(d, d, x[d], y[d]);
+      const mmr_context_stats st = hc->Stats();
+      return st.invariant_checks > 0 ? st.operation_hash : 0;
+    };
+    const int64_t h1 = run_schedule(false), h2 = run_schedule(false), h3 = run_schedule(true);
+    EXPECT(h1 != 0 && h1 == h2 && h1 != h3);
+  }
 
   std::printf("OK\n");
   return 0;

@@ -13,7 +13,9 @@
 #include <vector>
 
 #include "chunk_ops.h"
+#include "group_ops.h"
 #include "mmreshard.h"
+#include "planner.h"
 
 namespace {
 
@@ -74,6 +76,30 @@ struct HostMem {
   static void storeu(ptr p, T v) { put<T>(p, v, 1, "out-of-bounds store"); }
   static uintptr_t addr(ptr p) { return reinterpret_cast<uintptr_t>(p); }
   static uintptr_t caddr(cptr p) { return reinterpret_cast<uintptr_t>(p); }
+};
+
+// LDS of the span kernel: a host array; a cell read before it is written shows up as wrong bytes (poison).
+thread_local const uint8_t* g_lds_lo = nullptr;
+thread_local const uint8_t* g_lds_hi = nullptr;
+struct HostLds {
+  static bool ok(const uint8_t* p, size_t n) {
+    if (p >= g_lds_lo && p + n <= g_lds_hi) return true;
+    violation("LDS access outside the staging array", reinterpret_cast<uintptr_t>(p), n);
+    return false;
+  }
+  static void store16u(uint8_t* p, mmr::V16 v) {
+    if (ok(p, 16)) std::memcpy(p, &v, 16);
+  }
+  static void store8(uint8_t* p, uint8_t v) {
+    if (ok(p, 1)) *p = v;
+  }
+  static mmr::V16 load16(const uint8_t* p) {
+    mmr::V16 v{};
+    if (reinterpret_cast<uintptr_t>(p) % 16) violation("misaligned LDS vector load", reinterpret_cast<uintptr_t>(p), 16);
+    if (ok(p, 16)) std::memcpy(&v, p, 16);
+    return v;
+  }
+  static uint8_t load8(const uint8_t* p) { return ok(p, 1) ? *p : 0; }
 };
 
 template <typename T>
@@ -156,11 +182,113 @@ int mmr_emulate_plan(const mmr_plan* plan, void* const* slot_ptrs, const size_t*
     g_ranges.push_back(Range{p, p + slot_bytes[i]});
   }
   auto base = [&](uint32_t slot, uint64_t off) { return static_cast<uint8_t*>(slot_ptrs[slot]) + off; };
-  for (int kind = 0; kind < 2 && g_error.empty(); ++kind) {
-    const int64_t n = mmr_plan_get_copy_chunks(plan, kind, nullptr, 0);
+  for (const mmr::CopyPiece& pc : plan->copy_pieces)
+    if (pc.dst_slot >= n_slots || (pc.src_slot != MMR_SLOT_FILL && pc.src_slot >= n_slots))
+      g_error = "piece names a slot outside the pointer table";
+  for (const mmr::SpanMember& m : plan->span_members)
+    if (m.dst_slot >= n_slots) g_error = "span member names a slot outside the pointer table";
+  for (const mmr::SpanPiece& pc : plan->span_pieces)
+    if (pc.src_slot != MMR_SLOT_FILL && pc.src_slot >= n_slots) g_error = "span piece names a slot outside the pointer table";
+  const uint32_t mode = xcd_mode == 0 ? 64 : xcd_mode;
+  if (g_error.empty() && plan->n_copy_chunks) {
+    // the copy-group launch as the kernel runs it: the table bound to addresses, every workgroup decoding its chunk
+    std::vector<mmr::CopyPiece> pieces = plan->copy_pieces;
+    for (mmr::CopyPiece& pc : pieces) {
+      pc.dst = reinterpret_cast<uint64_t>(base(pc.dst_slot, pc.dst));
+      pc.src = pc.src_slot == MMR_SLOT_FILL ? 0 : reinterpret_cast<uint64_t>(base(pc.src_slot, pc.src));
+    }
+    const std::vector<uint32_t> hints = mmr::group_hints(plan->copy_groups, plan->n_copy_chunks);
+    for_each_chunk(plan->n_copy_chunks, mode, [&](uint32_t ci) {
+      const uint32_t gi = mmr::find_group(plan->copy_groups.data(), static_cast<uint32_t>(plan->copy_groups.size()),
+                                          (shape & 1) ? nullptr : hints.data(), ci);
+      const mmr::CopyGroup& g = plan->copy_groups[gi];
+      if (ci < g.first_chunk || ci - g.first_chunk >= g.n_chunks) {
+        g_error = "chunk " + std::to_string(ci) + " resolved to the wrong group";
+        return;
+      }
+      const mmr::DecodedCopy d = mmr::decode_copy(g, ci - g.first_chunk);
+      if (d.piece >= pieces.size() || d.n1 == 0 || d.n2 == 0) {
+        g_error = "chunk " + std::to_string(ci) + " decodes to nothing";
+        return;
+      }
+      const mmr::CopyPiece& pc = pieces[d.piece];
+      const mmr_copy_chunk c = mmr::copy_chunk_of(g, pc, d);
+      uint8_t* dst = reinterpret_cast<uint8_t*>(c.dst_off);
+      const uint8_t* src = c.src_slot == MMR_SLOT_FILL ? dst : reinterpret_cast<const uint8_t*>(c.src_off);
+      switch (shape) {  // 0 and 2 run the lean chunk code where the group allows it, 1 and 3 always the general one
+        case 1: run_copy16<128, 4>(c, src, dst); break;
+        case 2:
+          for (uint32_t tid = 0; tid < 512; ++tid) mmr::copy_group_rows<HostMem, 512, 1>(g, pc, c, src, dst, tid);
+          break;
+        case 3: run_copy16<64, 8>(c, src, dst); break;
+        default:
+          for (uint32_t tid = 0; tid < 256; ++tid) mmr::copy_group_rows<HostMem, 256, 2>(g, pc, c, src, dst, tid);
+          break;
+      }
+    });
+  }
+  if (g_error.empty() && plan->n_span_chunks) {
+    std::vector<mmr::SpanMember> members = plan->span_members;
+    std::vector<mmr::SpanPiece> pieces = plan->span_pieces;
+    for (mmr::SpanMember& m : members) m.dst = reinterpret_cast<uint64_t>(base(m.dst_slot, m.dst));
+    for (mmr::SpanPiece& pc : pieces)
+      pc.src = pc.src_slot == MMR_SLOT_FILL ? 0 : reinterpret_cast<uint64_t>(base(pc.src_slot, pc.src));
+    alignas(16) static thread_local uint8_t safe[16];
+    g_ranges.push_back(Range{reinterpret_cast<uintptr_t>(safe), reinterpret_cast<uintptr_t>(safe) + 16});
+    alignas(16) static thread_local uint8_t lds[mmr::kSpanLdsBytes];
+    g_lds_lo = lds;
+    g_lds_hi = lds + sizeof(lds);
+    const std::vector<uint32_t> hints = mmr::group_hints(plan->span_groups, plan->n_span_chunks);
+    for_each_chunk(plan->n_span_chunks, mode, [&](uint32_t ci) {
+      const uint32_t gi = mmr::find_group(plan->span_groups.data(), static_cast<uint32_t>(plan->span_groups.size()),
+                                          (shape & 1) ? nullptr : hints.data(), ci);
+      const mmr::SpanGroup& g = plan->span_groups[gi];
+      if (ci < g.first_chunk || ci - g.first_chunk >= g.n_chunks) {
+        g_error = "span chunk " + std::to_string(ci) + " resolved to the wrong group";
+        return;
+      }
+      uint32_t member, lm;
+      mmr::deinterleave(g.il, ci - g.first_chunk, &member, &lm);
+      if (member >= g.il.members || lm >= g.il.member_chunks) {
+        g_error = "span chunk " + std::to_string(ci) + " decodes outside its group";
+        return;
+      }
+      const mmr::SpanMember& m = members[g.first_member + member];
+      uint64_t x0;
+      uint32_t len;
+      mmr::span_range(g, lm, &x0, &len);
+      if (len == 0 || len > g.span || x0 + len > g.band_bytes) {
+        g_error = "span chunk " + std::to_string(ci) + " covers a bad range";
+        return;
+      }
+      uint8_t* dst = reinterpret_cast<uint8_t*>(m.dst + x0);
+      const uint32_t a = static_cast<uint32_t>(m.dst + x0) & 15u;
+      std::memset(lds, 0xA5 ^ static_cast<int>(ci & 0x3f), sizeof(lds));
+      // a phase runs for every thread before the next one starts: the workgroup barrier
+      switch (shape) {
+        case 1:
+          for (uint32_t tid = 0; tid < 128; ++tid) mmr::span_gather<HostMem, HostLds, 128, 4>(g, m, pieces.data(), safe, x0, len, a, lds, tid);
+          for (uint32_t tid = 0; tid < 128; ++tid) mmr::span_write<HostMem, HostLds, 128, 4>(dst, len, a, lds, tid);
+          break;
+        case 2:
+          for (uint32_t tid = 0; tid < 256; ++tid) mmr::span_gather<HostMem, HostLds, 256, 1>(g, m, pieces.data(), safe, x0, len, a, lds, tid);
+          for (uint32_t tid = 0; tid < 256; ++tid) mmr::span_write<HostMem, HostLds, 256, 1>(dst, len, a, lds, tid);
+          break;
+        case 3:
+          for (uint32_t tid = 0; tid < 512; ++tid) mmr::span_gather<HostMem, HostLds, 512, 3>(g, m, pieces.data(), safe, x0, len, a, lds, tid);
+          for (uint32_t tid = 0; tid < 512; ++tid) mmr::span_write<HostMem, HostLds, 512, 3>(dst, len, a, lds, tid);
+          break;
+        default:
+          for (uint32_t tid = 0; tid < 256; ++tid) mmr::span_gather<HostMem, HostLds, 256, 2>(g, m, pieces.data(), safe, x0, len, a, lds, tid);
+          for (uint32_t tid = 0; tid < 256; ++tid) mmr::span_write<HostMem, HostLds, 256, 2>(dst, len, a, lds, tid);
+          break;
+      }
+    });
+  }
+  if (g_error.empty()) {
+    const int64_t n = mmr_plan_get_copy_chunks(plan, 1, nullptr, 0);
     std::vector<mmr_copy_chunk> chunks(static_cast<size_t>(n));
-    mmr_plan_get_copy_chunks(plan, kind, chunks.data(), n);
-    const uint32_t mode = kind == 0 ? (xcd_mode == 0 ? 64 : xcd_mode) : (xcd_mode == 0 ? 64 : xcd_mode);
+    mmr_plan_get_copy_chunks(plan, 1, chunks.data(), n);
     for_each_chunk(n, mode, [&](uint32_t ci) {
       const mmr_copy_chunk& c = chunks[ci];
       if (c.dst_slot >= n_slots || (c.src_slot != MMR_SLOT_FILL && c.src_slot >= n_slots)) {
@@ -169,22 +297,12 @@ int mmr_emulate_plan(const mmr_plan* plan, void* const* slot_ptrs, const size_t*
       }
       uint8_t* dst = base(c.dst_slot, c.dst_off);
       const uint8_t* src = c.src_slot == MMR_SLOT_FILL ? dst : base(c.src_slot, c.src_off);
-      if (kind == 0) {
-        if (c.align != 16) g_error = "chunk in the aligned table is not 16-byte aligned";
-        switch (shape) {
-          case 1: run_copy16<128, 4>(c, src, dst); break;
-          case 2: run_copy16<64, 8>(c, src, dst); break;
-          case 3: run_copy16<512, 1>(c, src, dst); break;
-          default: run_copy16<256, 2>(c, src, dst); break;
-        }
-      } else {
-        if (c.n2 != 1) g_error = "generic chunk with n2 != 1";
-        switch (shape) {
-          case 1: run_generic<128, 4>(c, src, dst); break;
-          case 2: run_generic<256, 1>(c, src, dst); break;
-          case 3: run_generic<256, 4>(c, src, dst); break;
-          default: run_generic<256, 2>(c, src, dst); break;
-        }
+      if (c.n2 != 1) g_error = "generic chunk with n2 != 1";
+      switch (shape) {
+        case 1: run_generic<128, 4>(c, src, dst); break;
+        case 2: run_generic<256, 1>(c, src, dst); break;
+        case 3: run_generic<256, 4>(c, src, dst); break;
+        default: run_generic<256, 2>(c, src, dst); break;
       }
     });
   }

@@ -27,7 +27,7 @@ def raw_global(a: dict, g: np.ndarray) -> np.ndarray:
 def apply_plan(plan: "mm.Plan", buffers: Sequence[np.ndarray]) -> None:
     """Executes a plan's tables on host buffers (one flat uint8 array per slot)
     exactly as the kernels define a chunk; pure NumPy, for CPU-side checks."""
-    for kind in (0, 1):
+    for kind in (0, 1, 2):  # copy-group chunks as decoded, generic chunks, the row pieces of the span groups
         for c in plan.copy_chunks(kind):
             dst = buffers[int(c["dst_slot"])]
             fill = int(c["src_slot"]) == 0xFFFFFFFF

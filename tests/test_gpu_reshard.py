@@ -315,33 +315,76 @@ def test_store_interface(ctx):
     assert after["cache_hits"] == before["cache_hits"] + 1
     assert after["bytes_allocated"] == before["bytes_allocated"]
     assert st2.unique_id > st.unique_id
+    ctx.ClearStoreCache()  # also empties the allocator's pool of freed stores: only st2 is left
+    assert ctx.stats["bytes_allocated"] >= 4 * 4096
+    held = ctx.stats["bytes_allocated"]
     ctx.Free(st2, keep_in_cache=True)
+    assert ctx.stats["bytes_allocated"] == held  # parked, not released
     ctx.ClearStoreCache()
-    assert ctx.stats["bytes_allocated"] == before["bytes_allocated"] - 4 * 4096
+    assert ctx.stats["bytes_allocated"] == held - 4 * 4096
+    # a store freed without keep_in_cache goes to the allocator's pool; the next store of its size takes it back
+    st3 = ctx.CreateStore(shape, name="acts3")
+    allocs = ctx.stats["device_allocations"]
+    ctx.Free(st3)
+    st4 = ctx.CreateStore(mm.sharded_shape("S32", [(32, 2, 0), (4, 2, 1)], 7, 4), name="other type, same bytes")
+    assert ctx.stats["device_allocations"] == allocs and ctx.stats["pool_hits"] >= 1
+    assert ctx.ReadShard(st4, 7).tobytes() == bytes(32 * 4)  # zero-filled again
+    ctx.Free(st4)
 
 
 def test_plan_and_binding_caches(ctx):
-    """One plan per descriptor pair (keyed like ReshardKey), one pointer table per store pair."""
+    """One plan per descriptor pair (keyed like ReshardKey).  The first launch on a set of buffers carries its table
+    in the kernel's argument block, the second one builds the device tables for those buffers, later ones find
+    them; none of it makes the calling thread wait for the device."""
     s_shape = mm.sharded_shape("BF16", [(64, 1, 0), (256, 4, 1)], 0, 4)
     d_shape = mm.sharded_shape("BF16", [(64, 2, 0), (256, 1, 1)], 4, 2)
     a, b = ctx.CreateStore(s_shape), ctx.CreateStore(d_shape)
     c, d = ctx.CreateStore(s_shape), ctx.CreateStore(d_shape)
     s0 = ctx.stats
-    ctx.Reshard(a, b)
-    ctx.Reshard(a, b)
-    ctx.Reshard(c, d)
+    ctx.Reshard(a, b)   # argument block
+    ctx.Reshard(a, b)   # builds the device tables
+    ctx.Reshard(a, b)   # finds them
+    ctx.Reshard(c, d)   # other buffers: argument block again, same plan
     ctx.Sync()
     s1 = ctx.stats
     assert s1["plans_built"] - s0["plans_built"] == 1
-    assert s1["bindings_built"] - s0["bindings_built"] == 2
+    assert s1["plan_cache_hits"] - s0["plan_cache_hits"] == 3
+    assert s1["inline_launches"] - s0["inline_launches"] == 2
+    assert s1["bindings_built"] - s0["bindings_built"] == 1
     assert s1["binding_cache_hits"] - s0["binding_cache_hits"] == 1
-    assert s1["reshard_calls"] - s0["reshard_calls"] == 3
+    assert s1["reshard_calls"] - s0["reshard_calls"] == 4
+    assert s1["host_blocking_syncs"] == s0["host_blocking_syncs"]
     with pytest.raises(mm.MmrError):
         ctx.Reshard(a, a)
     with pytest.raises(mm.MmrError):
         ctx.Reshard(a, ctx.CreateStore(mm.sharded_shape("BF16", [(64, 2, 0), (128, 1, 1)], 4, 2)))
     for st in (a, b, c, d):
         ctx.Free(st)
+
+
+def test_first_reshard_of_a_pair_does_not_wait_for_the_device():
+    """A plain Reshard on descriptors never seen before plans, binds and launches without a single blocking
+    synchronisation (the reference's Reshard is asynchronous), whichever launch classes the plan has; the plan it
+    builds is the same on every run (nothing is timed unless TuneReshard is called)."""
+    for index, scale in ((2, 8), (5, 8), (13, 8), (4, 16)):
+        arrays = workloads.config(index, scale)
+        gs = [workloads.generate(a) for a in arrays]
+        seen = []
+        for _ in range(2):
+            with mm.ReshardContext(0) as ctx:
+                srcs, dsts = make_stores(ctx, arrays, gs)
+                ctx.Sync()
+                before = ctx.stats
+                ctx.ReshardBatch(srcs, dsts)
+                after = ctx.stats
+                assert after["host_blocking_syncs"] == before["host_blocking_syncs"], index
+                assert after["plans_built"] == before["plans_built"] + 1
+                ctx.Sync()
+                _compare(arrays, gs, [read_all(ctx, d) for d in dsts])
+                st = ctx.batch_plan_stats(srcs, dsts)
+                assert st["orders_timed"] == 0
+                seen.append(st)
+        assert seen[0] == seen[1]
 
 
 def test_reshard_is_stream_ordered_after_assemble(ctx):
@@ -382,31 +425,49 @@ def test_adopted_buffers_are_used_in_place(ctx):
 
 
 def test_offload_to_host_and_back(ctx):
-    """OffloadDtoH / OffloadHtoD with pinned host memory; the mock's invariant that an
-    offloaded store cannot take part in device work (mm_mock_mm_xla.cc:347-356)."""
+    """OffloadDtoH / OffloadHtoD: asynchronous copies between the device cache and a host cache of pinned buffers
+    (zuku_execute_context_impl.cc:162-211); the mock's invariant that an offloaded store cannot take part in device
+    work (mm_mock_mm_xla.cc:347-356).  Neither call makes the host wait, and the second offload of a descriptor is
+    served from the host cache."""
     a = workloads.config(1, 8)[0]
     g = workloads.generate(a)
     srcs, dsts = make_stores(ctx, [a], [g])
+    ctx.Sync()
     s0 = ctx.stats
     ctx.OffloadDtoH([srcs[0]])
     s1 = ctx.stats
     assert ctx.IsOffloaded(srcs[0])
-    assert s1["bytes_allocated"] < s0["bytes_allocated"]
-    assert s1["host_bytes_allocated"] == s0["bytes_allocated"] - s1["bytes_allocated"]
+    assert s1["host_blocking_syncs"] == s0["host_blocking_syncs"]
+    assert s1["host_bytes_allocated"] > s0["host_bytes_allocated"]
+    assert s1["bytes_allocated"] == s0["bytes_allocated"]  # the device buffer is parked in the device cache
     with pytest.raises(mm.MmrError) as e:
         ctx.Reshard(srcs[0], dsts[0])
     assert "offloaded" in str(e.value)
     with pytest.raises(mm.MmrError):
         ctx.SliceLocalShard(srcs[0].devices[0], srcs[0])
     host_view = ctx.ReadShard(srcs[0], srcs[0].devices[1])  # reading back still works
+    expect = ro.make_shards(raw_global(a, g), oracle_shape(a["type"], a["src"]))
+    assert host_view.tobytes() == expect[srcs[0].devices[1]].tobytes()
+    s1 = ctx.stats
     ctx.OffloadHtoD([srcs[0]])
+    ctx.Reshard(srcs[0], dsts[0])  # offload -> reload -> reshard, all stream-ordered, no host wait
+    s2 = ctx.stats
     assert not ctx.IsOffloaded(srcs[0])
-    assert ctx.stats["host_bytes_allocated"] == 0 and ctx.stats["bytes_allocated"] == s0["bytes_allocated"]
-    assert ctx.ReadShard(srcs[0], srcs[0].devices[1]).tobytes() == host_view.tobytes()
-    ctx.Reshard(srcs[0], dsts[0])
+    assert s2["host_blocking_syncs"] == s1["host_blocking_syncs"]
+    assert s2["cache_hits"] == s1["cache_hits"] + 1 and s2["device_allocations"] == s1["device_allocations"]
     ctx.Sync()
     _compare([a], [g], [read_all(ctx, dsts[0])])
+    # a second offload of the same descriptor: the pinned buffer comes from the host cache
+    ctx.OffloadDtoH([srcs[0]])
+    s3 = ctx.stats
+    assert s3["host_cache_hits"] == s2["host_cache_hits"] + 1
+    assert s3["host_bytes_allocated"] == s2["host_bytes_allocated"]
+    ctx.OffloadHtoD([srcs[0]])
+    ctx.Sync()
+    assert ctx.ReadShard(srcs[0], srcs[0].devices[1]).tobytes() == host_view.tobytes()
     ctx.Free(srcs[0]); ctx.Free(dsts[0])
+    ctx.ClearStoreCache()
+    assert ctx.stats["host_bytes_allocated"] == s0["host_bytes_allocated"]
 
 
 def test_plan_prepared_before_the_first_reshard(ctx):
@@ -511,23 +572,26 @@ def test_reshard_replays_from_a_hip_graph():
         ctx.close()
 
 
-def test_table_order_is_tuned_on_first_use_and_results_do_not_change():
-    """The first reshard of a descriptor pair times a few table orders on the caller's
-    buffers and keeps the fastest; whichever wins, the bytes are the oracle's.  A fixed
-    order or MMR_PLAN_NO_AUTOTUNE switches the tuning off."""
+def test_table_order_is_tuned_on_request_and_results_do_not_change():
+    """TuneReshard times a few launch orders on the caller's buffers and keeps the fastest; whichever wins, the
+    bytes are the oracle's.  Nothing is timed without it, and a fixed order leaves nothing to time."""
     arrays = workloads.config(3, 2)  # 4,096 aligned chunks
     gs = [workloads.generate(a) for a in arrays]
-    for flags, order, tuned in ((0, 0, True), (2, 0, False), (0, 2, False)):
+    for order, tuned in ((0, True), (2, False)):
         ctx = mm.ReshardContext(0)
         try:
-            ctx.set_plan_options(0, order, 0, flags)
+            ctx.set_plan_options(0, order, 0, 0)
             outs, srcs, dsts = gpu_reshard(ctx, arrays, gs, keep=True)
             _compare(arrays, gs, outs)
+            assert ctx.plan_stats(srcs[0], dsts[0])["orders_timed"] == 0
+            syncs = ctx.stats["host_blocking_syncs"]
+            used = ctx.TuneReshard(srcs[0], dsts[0])
             st = ctx.plan_stats(srcs[0], dsts[0])
-            say("flags %d order %d: %d orders timed, order used %d / %d KiB" % (
-                flags, order, st["orders_timed"], st["order_used"], st["interleave_kib"]))
-            assert (st["orders_timed"] >= 2) == tuned
-            # a second reshard of the same stores reuses the tuned plan: no further timing, same bytes
+            say("order %d: %d orders timed, order used %d / %d KiB" % (order, st["orders_timed"], st["order_used"],
+                                                                        st["interleave_kib"]))
+            assert (st["orders_timed"] >= 2) == tuned and used == st["order_used"]
+            assert (ctx.stats["host_blocking_syncs"] > syncs) == tuned
+            # later reshards of the same stores use the kept plan: one launch, same bytes
             before = ctx.stats["kernel_launches"]
             ctx.Reshard(srcs[0], dsts[0])
             ctx.Sync()

@@ -172,14 +172,15 @@ def test_plan_rejects_mismatched_pairs():
 
 
 def test_generic_chunks_are_bounded_in_lane_work_as_well_as_in_bytes():
-    """The generic kernel spends one lane per (row, 16-byte slot) pair: the one-byte pad
-    column of configuration 5's last tile must not come out as chunks of thousands of
-    rows (each would keep one workgroup busy long after the rest of the launch)."""
+    """The generic kernel (ragged boxes the span kernel does not take; forced here with MMR_PLAN_NO_SPAN) spends
+    one lane per (row, 16-byte slot) pair: the one-byte pad column of configuration 5's last tile must not come out
+    as chunks of thousands of rows (each would keep one workgroup busy long after the rest of the launch)."""
+    from multimesh_jax_amd import _binding as B
     arrays = workloads.config(5)
     plan = mm.Plan([lib_shape(a["type"], a["src"]) for a in arrays],
-                   [lib_shape(a["type"], a["dst"]) for a in arrays])
+                   [lib_shape(a["type"], a["dst"]) for a in arrays], flags=B.MMR_PLAN_NO_SPAN)
     g = plan.copy_chunks(1)
-    assert len(g) > 0 and len(plan.copy_chunks(0)) == 0
+    assert len(g) > 0 and len(plan.copy_chunks(0)) == 0 and plan.stats["n_span_chunks"] == 0
     slots = (g["w"].astype(np.int64) + 15) // 16 + 1
     pairs = g["n1"].astype(np.int64) * g["n2"] * slots
     assert pairs.max() <= 768
@@ -190,6 +191,41 @@ def test_generic_chunks_are_bounded_in_lane_work_as_well_as_in_bytes():
     # whole rows of 820 bytes: 6 to a chunk at this plan's size (45 MB -> ~5.4 KiB chunks), 8 (7 KiB) on a plan 8 times larger
     assert int(g[g["w"] == 820]["n1"].max()) == 6
     big = workloads.config(10)
-    plan_big = mm.Plan([lib_shape(a["type"], a["src"]) for a in big], [lib_shape(a["type"], a["dst"]) for a in big])
+    plan_big = mm.Plan([lib_shape(a["type"], a["src"]) for a in big], [lib_shape(a["type"], a["dst"]) for a in big],
+                       flags=B.MMR_PLAN_NO_SPAN)
     gb = plan_big.copy_chunks(1)
     assert int(gb[gb["w"] == 820]["n1"].max()) == 8
+
+
+def test_ragged_rows_become_destination_spans():
+    """Configuration 5 (4099-byte fp8 rows and 4097 x 4-byte rows, 3-way -> 5-way): every destination tile is one
+    dense band of rows whose pieces tile the row, cut into 128-byte aligned spans; the five tiles of an array are
+    interleaved in one group; the whole plan is two group records."""
+    arrays = workloads.config(5)
+    plan = mm.Plan([lib_shape(a["type"], a["src"]) for a in arrays],
+                   [lib_shape(a["type"], a["dst"]) for a in arrays])
+    s = plan.stats
+    assert s["n_copy16_chunks"] == 0 and s["n_copy_generic_chunks"] == 0 and s["n_transpose_chunks"] == 0
+    assert s["n_groups"] == 2  # one per array, five interleaved tiles each
+    # destination shards of 8 x 3280 and 11008 x 820 bytes, five each, in spans of 8 KiB
+    assert s["n_span_chunks"] == 5 * (-(-8 * 3280 // 8192)) + 5 * (-(-11008 * 820 // 8192))
+    assert s["table_bytes"] < 4096
+    pieces = plan.copy_chunks(2)
+    fp8 = pieces[pieces["d1"] == 820]
+    assert sorted(fp8["w"].tolist()) == sorted([820, 547, 273, 820, 274, 546, 819, 1])
+    assert (fp8["n1"].astype(np.int64) * fp8["n2"] == 11008).all()
+    assert int(fp8[fp8["src_slot"] == 0xFFFFFFFF]["w"].sum()) == 1  # the pad column of the last tile
+    assert s["bytes_moved"] == 8 * 4097 * 4 + 11008 * 4099 and s["bytes_filled"] == 8 * 3 * 4 + 11008
+
+
+def test_plan_tables_are_a_handful_of_records():
+    """The plan of the headline configuration: 4 groups (one per destination tile) of 8 pieces each; a 195-array
+    batch stays in the hundreds of KiB."""
+    a = workloads.config(2)[0]
+    plan = mm.Plan(lib_shape(a["type"], a["src"]), lib_shape(a["type"], a["dst"]))
+    s = plan.stats
+    assert s["n_groups"] == 4 and s["n_pieces"] == 32 and s["n_copy16_chunks"] == 65536
+    assert s["table_bytes"] < 8192
+    arrays = workloads.config(4)
+    plan4 = mm.Plan([lib_shape(a["type"], a["src"]) for a in arrays], [lib_shape(a["type"], a["dst"]) for a in arrays])
+    assert plan4.stats["table_bytes"] < 1 << 20

@@ -44,8 +44,8 @@ def _assert_equal(arrays, ref, got):
 
 def test_static_entry_point_matches_batch_on_two_calls_in_a_row():
     with mm.ReshardContext(0) as ctx:
-        # first call: configuration 2 at 1/2 scale (aligned chunks, 16,384 of them) together with the ragged arrays of
-        # configuration 5 at 1/8 scale (generic chunks and pad fills) and a transposed layout (tile chunks)
+        # first call: configuration 2 at 1/2 scale (copy groups, 16,384 chunks) together with the ragged arrays of
+        # configuration 5 at 1/8 scale (span groups with pad fills) and a transposed layout (tile chunks)
         first = workloads.config(2, 2) + workloads.config(5, 8) + workloads.config(13, 8)
         say("static entry point, first call: %d arrays" % len(first))
         ref, got, before, after = _both_ways(ctx, first)
@@ -63,7 +63,10 @@ def test_static_entry_point_matches_batch_on_two_calls_in_a_row():
 
 def test_static_entry_point_refuses_plans_beyond_the_array():
     with mm.ReshardContext(0) as ctx:
-        arrays = workloads.config(4, 2)  # 195 arrays, ~160k chunks: more than 8 MiB of tables
+        # ragged rows lowered to one record per workgroup (the span kernel switched off): ~36,000 records of 72 bytes,
+        # more than the array holds
+        ctx.set_plan_options(0, 0, 0, B.MMR_PLAN_NO_SPAN)
+        arrays = workloads.config(10, 2)
         gs = [workloads.generate(a) for a in arrays]
         srcs, dsts = make_stores(ctx, arrays, gs, poison=None)
         say("static entry point, oversized plan")
