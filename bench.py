@@ -35,9 +35,9 @@ if ROOT not in sys.path:
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
-# FETCH_SIZE reads low by this factor, WRITE_SIZE by none: what the two counters report (KiB) for a 512 MiB device
-# copy of known size, measured with the runtime's own hipMemcpyDtoD kernel and with this library's copy kernel
-FETCH_SCALE, WRITE_SCALE = 1.969, 1.000
+# What the two counters report (KiB per dispatch) for a 512 MiB device-to-device copy by the HIP runtime's own kernel
+# (__amd_rocclr_copyBuffer, `bench.py --calibrate-copy`): FETCH_SIZE 262,155.5 -> x 2.000, WRITE_SIZE 524,288.0 -> x 1.000
+FETCH_SCALE, WRITE_SCALE = 2.000, 1.000
 
 
 def kernel_sources_digest():
@@ -297,6 +297,10 @@ def main():
                     help="keep the planner's default launch order instead of timing a few on the first buffer set")
     ap.add_argument("--unbatched", action="store_true",
                     help="multi-array configurations: one Reshard call per array instead of one batched call (probing)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="instead of a reshard, copy 512 MiB device to device with the HIP runtime's own copy kernel a few "
+                         "times (run under rocprofv3 --pmc FETCH_SIZE or WRITE_SIZE: the counters' factors for a kernel "
+                         "that is not this library's)")
     ap.add_argument("--record-traffic", type=str, default="",
                     help="directory with FETCH_SIZE/ and WRITE_SIZE/ rocprofv3 --pmc outputs of --config: writes "
                          "profiles/traffic_config<c>.json and exits (needs no GPU)")
@@ -323,6 +327,18 @@ def main():
     from gpu_helpers import read_all
 
     ctx = mm.ReshardContext(0)
+    if args.calibrate_copy:
+        shape = (8, 4096, 8192)
+        a = mm.sharded_shape("BF16", [(n, 1, i) for i, n in enumerate(shape)], 0, 1)
+        b = mm.sharded_shape("BF16", [(n, 1, i) for i, n in enumerate(shape)], 1, 1)
+        src, dst = ctx.CreateStore(a), ctx.CreateStore(b)
+        ptr = ctx.SliceLocalShard(0, src)
+        for _ in range(5):
+            ctx.AssembleShards(b, 1, ptr, existing_store=dst, size=512 << 20, where=3)
+        ctx.Sync()
+        print(json.dumps({"calibration": "5 x hipMemcpyAsync device to device of %d bytes" % (512 << 20)}))
+        ctx.close()
+        return
     if args.chunk_bytes or args.order or args.xcd_mode or args.flags:
         ctx.set_plan_options(args.chunk_bytes, args.order, args.xcd_mode, args.flags)
 

@@ -324,8 +324,11 @@ int mmr_clear_store_cache(mmr_context* ctx);
 /* AssembleShards / Shard{data, local_device_id, size},
  * zuku_execute_context.h:20-24,89-97, zuku_execute_context_impl.cc:384-424: one
  * flat copy of `size` bytes into the buffer of `device`.  data_on_device == 1:
- * `data` is a device pointer (stream-ordered copy); 0: host memory, consumed
- * before the call returns; 2: the HIP runtime decides which (blocking). */
+ * `data` is a device pointer (stream-ordered copy; large aligned shards go
+ * through the library's own copy kernel); 0: host memory, consumed before the
+ * call returns; 2: the HIP runtime tells which of the two; 3: a device pointer,
+ * always copied by the runtime's hipMemcpyAsync (the reference's MemcpyDtoDAsync
+ * as it is; also the independent kernel the traffic counters are calibrated on). */
 int mmr_store_assemble(mmr_context* ctx, mmr_store* store, int64_t device, const void* data, size_t size,
                        int32_t data_on_device);
 
@@ -400,6 +403,11 @@ int mmr_context_prepare(mmr_context* ctx, const mmr_sharded_shape* srcs, const m
  * context's stream waits for a caller's hipEvent_t / records one. */
 int mmr_context_wait_event(mmr_context* ctx, void* hip_event);
 int mmr_context_record_event(mmr_context* ctx, void* hip_event);
+
+/* RunAfterAllTasks, zuku_execute_context.h:53-54, zuku_execute_context_impl.cc:347-354: fn(arg) runs on a runtime
+ * thread once everything queued on the context's stream so far is done; the call itself does not wait.  fn must not
+ * call into this library. */
+int mmr_context_run_after(mmr_context* ctx, void (*fn)(void*), void* arg);
 
 /* Blocks until everything queued on the context's stream is done. */
 int mmr_sync(mmr_context* ctx);

@@ -167,6 +167,7 @@ PROTOTYPES = {
     "mmr_reshard_batch_static": (C.c_int, [VP, P(VP), P(VP), I32]),
     "mmr_reshard_bind": (C.c_int, [VP, P(VP), P(VP), I32]),
     "mmr_reshard_validate": (C.c_int, [VP, VP, VP]),
+    "mmr_context_run_after": (C.c_int, [VP, C.CFUNCTYPE(None, VP), VP]),
     "mmr_sync": (C.c_int, [VP]),
     "mmr_timer_start": (C.c_int, [VP]),
     "mmr_timer_stop": (C.c_int, [VP, P(C.c_float)]),
@@ -190,6 +191,25 @@ class MmrError(RuntimeError):
 _lib = None
 
 
+def source_digest():
+    """Digest of the sources next to this file, computed as csrc/build.sh does; None where they are not there."""
+    import hashlib
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    names = sorted([os.path.join("include", n) for n in os.listdir(os.path.join(root, "include")) if n.endswith(".h")]
+                   + [os.path.join("multimesh-jax_amd", "csrc", n)
+                      for n in os.listdir(os.path.join(root, "multimesh-jax_amd", "csrc"))]) \
+        if os.path.isdir(os.path.join(root, "include")) and os.path.isdir(os.path.join(root, "multimesh-jax_amd", "csrc")) else None
+    if not names:
+        return None
+    h = hashlib.sha256()
+    for n in names:
+        h.update(n.encode() + b"\n")
+        with open(os.path.join(root, n), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
 def load():
     """Loads libmmreshard.so and types every entry point. Raises if it is not built."""
     global _lib
@@ -203,6 +223,12 @@ def load():
             fn = getattr(lib, name)
             fn.restype = restype
             fn.argtypes = argtypes
+        built_from = lib.mmr_version().decode().rsplit(" ", 1)[-1]
+        here = source_digest()
+        if here is not None and built_from != here:
+            raise ImportError(
+                "%s was built from other sources (digest %s) than the ones next to it (%s): rebuild it with "
+                "multimesh-jax_amd/csrc/build.sh" % (LIB_PATH, built_from, here))
         _lib = lib
     return _lib
 

@@ -373,7 +373,8 @@ class ReshardContext:
     def AssembleShards(self, shape: B.ShardedShape, device: int, data, existing_store: Optional[StoreHandle] = None,
                        size: Optional[int] = None, where: int = 1) -> StoreHandle:
         """Shard{data, local_device_id, size}: `data` is a NumPy array (host) or an int pointer; `where` says what an
-        int pointer points at: 1 device memory, 0 host memory, 2 let the runtime find out."""
+        int pointer points at: 1 device memory, 0 host memory, 2 let the runtime find out, 3 device memory copied by
+        the runtime's own kernel."""
         store = existing_store if existing_store is not None else self.CreateStore(shape)
         if isinstance(data, np.ndarray):
             arr = np.ascontiguousarray(data)

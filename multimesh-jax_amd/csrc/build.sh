@@ -2,10 +2,12 @@
 # Builds libmmreshard.so (C ABI + gfx950 kernels) next to the Python package.
 set -euo pipefail
 here="$(cd "$(dirname "${BASH_SOURCE[0]}")" && pwd)"
+# digest of everything the library is built from (file names and contents, sorted): mmr_version() reports it
+digest="$(cd "${here}/../.." && for f in $(ls include/*.h multimesh-jax_amd/csrc/* | LC_ALL=C sort); do echo "$f"; cat "$f"; done | sha256sum | cut -c1-16)"
 out="${MMR_BUILD_OUT:-${here}/../libmmreshard.so}"  # MMR_BUILD_OUT / MMR_BUILD_FLAGS: tuning builds
 hipcc --offload-arch=gfx950 -O3 -std=c++17 -fPIC -shared \
   -Xclang -target-feature -Xclang -packed-fp32-ops \
-  -Wall -Wextra -Wno-unused-command-line-argument ${MMR_BUILD_FLAGS:-} \
+  -Wall -Wextra -Wno-unused-command-line-argument ${MMR_BUILD_FLAGS:-} -DMMR_SOURCE_DIGEST="\"${digest}\"" \
   -I"${here}/../../include" -I"${here}" \
   "${here}/geometry.cc" "${here}/sharding_frontend.cc" "${here}/planner.cc" \
   "${here}/context.cc" "${here}/hip_execute_context.cc" "${here}/shard_buffer.cc" "${here}/kernels.hip" \

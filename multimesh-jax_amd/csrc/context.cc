@@ -696,7 +696,7 @@ int tune_locked(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts
   struct Candidate {
     uint32_t order, kib;
   };
-  const Candidate candidates[] = {{4, 64}, {4, 1024}, {4, 4096}, {2, 0}};
+  const Candidate candidates[] = {{4, 64}, {4, 512}, {4, 2048}, {4, 4096}, {2, 0}};
   std::unique_ptr<DevicePlan> best;
   for (const Candidate& cand : candidates) {
     mmr_plan_options o = base;
@@ -1033,6 +1033,8 @@ int mmr_store_assemble(mmr_context* ctx, mmr_store* store, int64_t device, const
   if (int rc = use_device(ctx)) return rc;
   // one flat copy of the shard's bytes, as AssembleShardsImpl does
   // (zuku_execute_context_impl.cc:405-415)
+  const bool runtime_copy = data_on_device == 3;  // a device pointer, copied by the runtime's own kernel
+  if (runtime_copy) data_on_device = 1;
   const hipMemcpyKind kind = data_on_device == 1   ? hipMemcpyDeviceToDevice
                              : data_on_device == 0 ? hipMemcpyHostToDevice
                                                    : hipMemcpyDefault;  // the runtime looks the pointer up
@@ -1048,7 +1050,7 @@ int mmr_store_assemble(mmr_context* ctx, mmr_store* store, int64_t device, const
   // a large device-resident shard goes through the library's own copy kernel (6.4 TB/s against 5.3 TB/s for the
   // runtime's device-to-device copy on MI355X); anything else through the runtime
   const uintptr_t bits = reinterpret_cast<uintptr_t>(data) | reinterpret_cast<uintptr_t>(store->tile(k));
-  if (data_on_device == 1 && size >= (1u << 20) && (bits & 15u) == 0) {
+  if (data_on_device == 1 && !runtime_copy && size >= (1u << 20) && (bits & 15u) == 0) {
     const size_t body = size & ~static_cast<size_t>(15);
     MMR_HIP(mmr::launch_flat_copy(data, store->tile(k), body, ctx->stream));
     ctx->stats.kernel_launches += 1;
@@ -1273,6 +1275,13 @@ int mmr_reshard_bind(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const*
   if (!ctx || n < 0 || (n > 0 && (!srcs || !dsts))) return fail(MMR_INVALID_ARGUMENT, "bad batch arguments");
   std::lock_guard<std::mutex> lock(ctx->mu);
   return reshard_locked(ctx, srcs, dsts, n, /*launch=*/false);
+}
+
+int mmr_context_run_after(mmr_context* ctx, void (*fn)(void*), void* arg) {
+  if (!ctx || !fn) return fail(MMR_INVALID_ARGUMENT, "null argument");
+  MMR_HIP(hipSetDevice(ctx->device));
+  MMR_HIP(hipLaunchHostFunc(ctx->stream, fn, arg));
+  return MMR_OK;
 }
 
 int mmr_sync(mmr_context* ctx) {

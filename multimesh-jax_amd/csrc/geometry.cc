@@ -123,7 +123,12 @@ using mmr::fail;
 extern "C" {
 
 const char* mmr_last_error(void) { return mmr::last_error(); }
-const char* mmr_version(void) { return "mmreshard 0.1 (gfx950)"; }
+#ifndef MMR_SOURCE_DIGEST
+#define MMR_SOURCE_DIGEST "unknown"
+#endif
+// "mmreshard <version> (gfx950) sources <digest>": the digest of the sources this binary was built from, so that a
+// loader can tell a stale binary from a current one.
+const char* mmr_version(void) { return "mmreshard 0.2 (gfx950) sources " MMR_SOURCE_DIGEST; }
 int mmr_itemsize(int32_t dtype) { return mmr::itemsize_of(dtype); }
 
 int mmr_validate_sharded_shape(const mmr_sharded_shape* s) {

@@ -268,6 +268,14 @@ void* HipExecuteContext::SliceLocalShard(int64_t local_device_id, const StoreHan
   return ptr;
 }
 
+void* HipExecuteContext::TilePointer(const StoreHandle& handle) {
+  require_live(handle, "TilePointer");
+  Flush();
+  void* ptr = nullptr;
+  check(mmr_store_shard_ptr_async(ctx_, handle.impl->array->store, handle.impl->global_device_id, &ptr), "TilePointer");
+  return ptr;
+}
+
 void HipExecuteContext::CopyShardToHost(const StoreHandle& handle, void* host_dst, size_t size) {
   require_live(handle, "CopyShardToHost");
   Flush();
@@ -348,9 +356,22 @@ void HipExecuteContext::CloseWindow() { Flush(); }
 
 void HipExecuteContext::RunAfterAllTasks(int64_t local_device_id, std::function<void()> on_done) {
   (void)local_device_id;
+  if (!on_done) return;  // zuku_execute_context_impl.cc:349
   Flush();
-  check(mmr_sync(ctx_), "RunAfterAllTasks");
-  on_done();
+  // deferred behind everything queued so far, like after(last_execute_events_[...]).defer(callback); the caller
+  // does not wait
+  auto* boxed = new std::function<void()>(std::move(on_done));
+  const int rc = mmr_context_run_after(
+      ctx_,
+      [](void* p) {
+        std::unique_ptr<std::function<void()>> fn(static_cast<std::function<void()>*>(p));
+        (*fn)();
+      },
+      boxed);
+  if (rc != MMR_OK) {
+    delete boxed;
+    check(rc, "RunAfterAllTasks");
+  }
 }
 
 void HipExecuteContext::MarkProfile(const std::string& name) { (void)name; }

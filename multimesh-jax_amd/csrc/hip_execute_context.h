@@ -165,6 +165,9 @@ class HipExecuteContext {
                              std::optional<StoreHandle> existing_store = std::nullopt);
   void Reshard(int64_t local_device_id, int64_t global_device_id, const StoreHandle& src, const StoreHandle& dst);
   void* SliceLocalShard(int64_t local_device_id, const StoreHandle& handle);
+  // The same pointer without waiting, for work that stays on the context's stream (an adapter that launches compute
+  // tasks there); queued reshards are issued first.
+  void* TilePointer(const StoreHandle& handle);
   ShardedShape GetStoreShardedShape(const StoreHandle& handle);
   bool HasLocalShard(const StoreHandle& handle);
   void Free(int64_t local_device_id, StoreHandle handle, bool keep_in_cache);

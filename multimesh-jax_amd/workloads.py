@@ -92,35 +92,11 @@ def config(index: int, scale: int = 1) -> List[dict]:
             _array("c5b_tokens", "S32", a, _side(a, (3, 1), 0), _side(a, (5, 1), 3), 5, "int32000"),
             _array("c5b_fp8", "F8E4M3FN", b, _side(b, (3, 1), 0), _side(b, (5, 1), 3), 6, "fp8"),
         ]
-    if index == 9:  # probe: configuration 2's sharding on an 8x larger array (4 GiB per side at scale 1)
-        shape = (64 // s, 4096, 8192)
-        return [_array("probe_big", "BF16", shape, _side(shape, (1, 1, 8), 0), _side(shape, (1, 4, 1), 8), 2, "raw")]
-    if index == 10:  # probe: configuration 5's fp8 array with 8x the rows
-        b = (88064 // s, 4099)
-        return [_array("probe_fp8_big", "F8E4M3FN", b, _side(b, (1, 3), 0), _side(b, (1, 5), 3), 6, "raw")]
-    if index == 11:  # probe: ragged rows, but every destination row comes from one source tile
-        b = (44032 // s, 4099)
-        return [_array("probe_fp8_1to5", "F8E4M3FN", b, _side(b, (1, 1), 0), _side(b, (1, 5), 3), 6, "raw")]
-    if index == 12:  # probe: ragged destination rows of 4-byte elements from one source tile
-        b = (44032 // s, 1025)
-        return [_array("probe_s32_1to5", "S32", b, _side(b, (1, 1), 0), _side(b, (1, 5), 3), 6, "raw")]
     if index in (13, 14, 15):  # transposed destination layout: rows 4-way, row-major -> columns 4-way, column-major
         type_ = {13: "BF16", 14: "F32", 15: "U8"}[index]
         shape = (8192 // s, 8192 // s)
         return [_array("transposed", type_, shape, _side(shape, (4, 1), 0),
                        _side(shape, (1, 4), 4, minor_to_major=(0, 1)), 13, "raw")]
-    if index == 16:  # probe: configuration 10's split with 16-byte aligned pieces (816 / 544 / 272-byte rows)
-        b = (88064 // s, 4080)
-        return [_array("probe_u8_aligned", "U8", b, _side(b, (1, 3), 0), _side(b, (1, 5), 3), 6, "raw")]
-    if index == 17:  # probe: byte-misaligned source rows (1387 bytes), destination rows of 832 bytes = 13 x 64
-        b = (88064 // s, 4160)
-        return [_array("probe_u8_dst64", "U8", b, _side(b, (1, 3), 0), _side(b, (1, 5), 3), 6, "raw")]
-    if index == 7:  # probe: 4-byte elements, uneven 3-way -> 5-way (dword-aligned, not 16-byte-aligned runs)
-        b = (11008 // s, 1025)
-        return [_array("probe_s32", "S32", b, _side(b, (1, 3), 0), _side(b, (1, 5), 3), 7, "raw")]
-    if index == 8:  # probe: 2-byte elements, uneven 3-way -> 5-way
-        b = (11008 // s, 2051)
-        return [_array("probe_u16", "U16", b, _side(b, (1, 3), 0), _side(b, (1, 5), 3), 8, "raw")]
     raise ValueError("configuration %r" % (index,))
 
 

@@ -5,6 +5,7 @@
 // restatement of the reshard (oracle/reshard_cpu.c), bit for bit.
 //
 // Needs a GPU.  Prints "OK" and exits 0 on success.
+#include <atomic>
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
@@ -132,6 +133,15 @@ static int run() {
     std::vector<uint16_t> got(expect[d - 8].size());
     ctx->CopyShardToHost(root[d], got.data(), got.size() * 2);
     EXPECT(std::memcmp(got.data(), expect[d - 8].data(), got.size() * 2) == 0);
+  }
+  // RunAfterAllTasks: the callback runs once the stream has drained, the call does not wait (a second reshard is
+  // queued right behind it)
+  {
+    std::atomic<int> fired{0};
+    ctx->RunAfterAllTasks(0, [&fired] { fired.fetch_add(1); });
+    ctx->RunAfterAllTasks(0, nullptr);  // no callback: nothing to do (zuku_execute_context_impl.cc:349)
+    EXPECT(mmr_sync(ctx->raw()) == MMR_OK);
+    EXPECT(fired.load() == 1);
   }
   // a device outside the store's device list has no shard to slice
   EXPECT(throws([&] { ctx->SliceLocalShard(0, root[0]); }, "holds no shard"));

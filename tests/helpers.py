@@ -12,6 +12,27 @@ from oracle import reshard_oracle as ro
 from oracle.sharding_oracle import ShardedShape, ShardingDim
 
 
+def test_config(index: int, scale: int = 1):
+    """The benchmark configurations of the package plus ragged shapes only the tests use."""
+    from multimesh_jax_amd import workloads as w
+
+    def one(name, type_, shape, src_tiles, dst_tiles, seed):
+        return [{"name": name, "type": type_, "shape": shape, "src": w.side(shape, src_tiles, 0),
+                 "dst": w.side(shape, dst_tiles, 3), "seed": seed, "dist": "raw"}]
+    if index == 7:  # 4-byte elements, uneven 3-way -> 5-way (dword-aligned, not 16-byte-aligned runs)
+        return one("ragged_s32", "S32", (11008 // scale, 1025), (1, 3), (1, 5), 7)
+    if index == 8:  # 2-byte elements, uneven 3-way -> 5-way
+        return one("ragged_u16", "U16", (11008 // scale, 2051), (1, 3), (1, 5), 8)
+    if index == 10:  # configuration 5's fp8 array with 8 times the rows
+        return one("ragged_fp8_big", "F8E4M3FN", (88064 // scale, 4099), (1, 3), (1, 5), 6)
+    if index == 11:  # ragged rows, every destination row from one source tile
+        return one("ragged_fp8_1to5", "F8E4M3FN", (44032 // scale, 4099), (1, 1), (1, 5), 6)
+    return w.config(index, scale)
+
+
+test_config.__test__ = False  # a helper, not a test
+
+
 def oracle_shape(type: str, side: dict) -> ShardedShape:
     return ShardedShape(type, tuple(ShardingDim(*d) for d in side["dims"]), side["dev_start"], side["dev_count"])
 

@@ -7,7 +7,7 @@ from hypothesis import given, settings, strategies as st
 
 from multimesh_jax_amd import workloads
 
-from helpers import oracle_outputs, run_plan_on_host
+from helpers import oracle_outputs, run_plan_on_host, test_config
 from test_planner_cpu import random_arrays
 
 
@@ -23,7 +23,7 @@ def _check(arrays, gs, **kw):
 @pytest.mark.parametrize("index,scale", [(1, 16), (2, 16), (3, 8), (5, 32), (6, 32), (7, 32), (8, 32), (11, 64)])
 @pytest.mark.parametrize("shape", [0, 1, 2, 3])
 def test_configs_through_the_kernel_code(index, scale, shape):
-    arrays = workloads.config(index, scale)
+    arrays = test_config(index, scale)
     gs = [workloads.generate(a) for a in arrays]
     _check(arrays, gs, shape=shape)
 

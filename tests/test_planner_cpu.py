@@ -8,7 +8,7 @@ from hypothesis import given, settings, strategies as st
 import multimesh_jax_amd as mm
 from multimesh_jax_amd import workloads
 
-from helpers import lib_shape, oracle_outputs, run_plan_on_host
+from helpers import lib_shape, oracle_outputs, run_plan_on_host, test_config
 
 
 def _check(arrays, globals_, **kw):
@@ -190,7 +190,7 @@ def test_generic_chunks_are_bounded_in_lane_work_as_well_as_in_bytes():
     assert int(fp8_pad["n1"].sum()) == 11008 and fp8_pad["n1"].max() <= 384
     # whole rows of 820 bytes: 6 to a chunk at this plan's size (45 MB -> ~5.4 KiB chunks), 8 (7 KiB) on a plan 8 times larger
     assert int(g[g["w"] == 820]["n1"].max()) == 6
-    big = workloads.config(10)
+    big = test_config(10)
     plan_big = mm.Plan([lib_shape(a["type"], a["src"]) for a in big], [lib_shape(a["type"], a["dst"]) for a in big],
                        flags=B.MMR_PLAN_NO_SPAN)
     gb = plan_big.copy_chunks(1)

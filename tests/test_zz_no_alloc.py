@@ -9,6 +9,7 @@ import multimesh_jax_amd as mm
 from multimesh_jax_amd import _binding as B, workloads
 
 from gpu_helpers import make_stores, read_all
+from helpers import test_config
 
 pytestmark = pytest.mark.gpu
 
@@ -66,7 +67,7 @@ def test_static_entry_point_refuses_plans_beyond_the_array():
         # ragged rows lowered to one record per workgroup (the span kernel switched off): ~36,000 records of 72 bytes,
         # more than the array holds
         ctx.set_plan_options(0, 0, 0, B.MMR_PLAN_NO_SPAN)
-        arrays = workloads.config(10, 2)
+        arrays = test_config(10, 2)
         gs = [workloads.generate(a) for a in arrays]
         srcs, dsts = make_stores(ctx, arrays, gs, poison=None)
         say("static entry point, oversized plan")
