@@ -209,6 +209,7 @@ typedef struct {
 #define MMR_PLAN_NO_AUTOTUNE 2u /* accepted and ignored: table orders are only timed on request (mmr_reshard_tune) */
 #define MMR_PLAN_NO_SPAN 4u     /* ragged boxes become generic chunks instead of span groups (testing) */
 #define MMR_PLAN_NO_INLINE 8u   /* group tables always live in device memory, never in the kernel's argument block */
+#define MMR_PLAN_NO_SEGMENT_TABLES 16u /* no span group uses the per-span table of (row, piece) pairs (testing) */
 
 typedef struct {
   uint32_t chunk_bytes; /* target bytes per copy chunk, 0 = default */

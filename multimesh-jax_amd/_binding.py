@@ -13,6 +13,7 @@ MMR_SLOT_FILL = 0xFFFFFFFF
 MMR_STORE_FROM_CACHE = 1
 MMR_STORE_UNINITIALIZED = 2
 MMR_PLAN_ALL_GENERIC, MMR_PLAN_NO_AUTOTUNE, MMR_PLAN_NO_SPAN = 1, 2, 4
+MMR_PLAN_NO_INLINE, MMR_PLAN_NO_SEGMENT_TABLES = 8, 16
 MMR_CHECK_INVARIANTS = 1
 MMR_STATIC_SCRATCH_BYTES = 1 << 20
 

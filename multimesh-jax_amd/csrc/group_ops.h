@@ -229,8 +229,11 @@ MMR_HD mmr_copy_chunk copy_chunk_of(const CopyGroup& g, const CopyPiece& p, cons
 // ---------------------------------------------------------------------------
 // Span groups
 // ---------------------------------------------------------------------------
-constexpr uint32_t kSpanMaxBytes = 16 * 1024;          // largest span a workgroup stages in LDS
-constexpr uint32_t kSpanLdsBytes = kSpanMaxBytes + 64;  // 16 spare bytes in front, up to 15 of phase, 16 + 16 spare behind
+constexpr uint32_t kSpanMaxBytes = 4 * 1024;           // largest span a workgroup (one wavefront) stages in LDS
+constexpr uint32_t kSpanLanes = 64, kSpanDepth = 4;     // the span kernel's launch shape: lanes x 16-byte vectors each
+constexpr uint32_t kSpanTablePieces = 4;                // most pieces per row of a group whose spans use a segment table
+constexpr uint32_t kSpanStageBytes = kSpanMaxBytes + 64;  // 16 spare bytes in front, up to 15 of phase, 16 + 16 spare behind
+constexpr uint32_t kSpanLdsBytes = kSpanStageBytes + kSpanLanes * 16;  // and a 16-byte segment record per lane
 constexpr uint32_t kSpanMaxRowBytes = 1u << 28;
 
 struct SpanPiece {
@@ -248,6 +251,9 @@ struct SpanMember {   // one destination tile's band
   uint32_t first_piece, k;  // pieces in ascending col order
   uint32_t wide;            // how many of them are wide
   FastDiv div_wide;         // by max(wide, 1)
+  uint32_t narrow;          // ... and how many narrower than 16 bytes
+  uint32_t reserved;
+  FastDiv div_k;
 };
 
 struct SpanGroup {
@@ -258,7 +264,8 @@ struct SpanGroup {
   uint32_t n1;          // rows per index of the slow row dim
   uint32_t span;        // bytes per chunk, a multiple of 128
   uint32_t head;        // bytes of the first chunk: the later ones start at multiples of `span` from the buffer's base
-  uint32_t reserved;
+  uint32_t table_mode;  // 1: at most kSpanTablePieces pieces per row and at most kSpanLanes (row, piece) pairs touch a
+                        // span: the lanes work those pairs out once, one each (span_table_build / span_table_gather)
   FastDiv div_W, div_n1;
   Interleave il;
 };
@@ -331,6 +338,29 @@ MMR_HD void span_item(const SpanGroup& g, const SpanPick& pk, uint32_t r0, uint3
   *at = static_cast<uint32_t>(16 + static_cast<int32_t>(a) + drel);
 }
 
+// The pieces narrower than 16 bytes of the rows that touch the span (uniform loop over the pieces): one byte per item.
+template <class M, class L, int THREADS>
+MMR_HD void span_gather_narrow(const SpanGroup& g, const SpanPiece* pc, uint32_t k, uint32_t nrows, uint32_t r0,
+                               uint32_t o0, int32_t ilen, uint32_t a, uint8_t* lds, uint32_t tid) {
+  for (uint32_t p = 0; p < k; ++p) {
+    const SpanPiece& c = pc[p];
+    if (c.w >= 16) continue;
+    const uint32_t total_n = nrows * c.w;
+    for (uint32_t i = tid; i < total_n; i += THREADS) {
+      const uint32_t r = i / c.w, b = i - r * c.w;
+      const int32_t drel = static_cast<int32_t>(r * g.W + c.col + b) - static_cast<int32_t>(o0);
+      if (drel < 0 || drel >= ilen) continue;
+      uint8_t value = 0;
+      if (c.src_slot != MMR_SLOT_FILL) {
+        const uint32_t row = r0 + r;
+        const uint32_t r2 = fdiv(row, g.div_n1), r1 = row - r2 * g.n1;
+        value = M::template loadu<uint8_t>(reinterpret_cast<typename M::cptr>(c.src) + (r2 * c.s2 + r1 * c.s1 + static_cast<int64_t>(b)));
+      }
+      L::store8(lds + 16 + a + static_cast<uint32_t>(drel), value);
+    }
+  }
+}
+
 template <class M, class L, int THREADS, int UNROLL>
 MMR_HD void span_gather(const SpanGroup& g, const SpanMember& m, const SpanPiece* pieces, typename M::cptr safe,
                         uint64_t x0, uint32_t len, uint32_t a, uint8_t* lds, uint32_t tid) {
@@ -388,22 +418,122 @@ MMR_HD void span_gather(const SpanGroup& g, const SpanMember& m, const SpanPiece
     for (int u = 0; u <= UNROLL; ++u)
       if (live[u]) L::store16u(lds + at[u], zero[u] ? V16{0, 0, 0, 0} : v[u]);
   }
-  for (uint32_t p = 0; p < k; ++p) {  // narrow pieces (uniform over the workgroup): one byte per item
-    const SpanPiece& c = pc[p];
-    if (c.w >= 16) continue;
-    const uint32_t total_n = nrows * c.w;
-    for (uint32_t i = tid; i < total_n; i += THREADS) {
-      const uint32_t r = i / c.w, b = i - r * c.w;
-      const int32_t drel = static_cast<int32_t>(r * W + c.col + b) - static_cast<int32_t>(o0);
-      if (drel < 0 || drel >= ilen) continue;
-      uint8_t value = 0;
-      if (c.src_slot != MMR_SLOT_FILL) {
-        const uint32_t row = r0 + r;
-        const uint32_t r2 = fdiv(row, g.div_n1), r1 = row - r2 * g.n1;
-        value = M::template loadu<uint8_t>(reinterpret_cast<typename M::cptr>(c.src) + (r2 * c.s2 + r1 * c.s1 + static_cast<int64_t>(b)));
-      }
-      L::store8(lds + 16 + a + static_cast<uint32_t>(drel), value);
+  if (m.narrow) span_gather_narrow<M, L, THREADS>(g, pc, k, nrows, r0, o0, ilen, a, lds, tid);
+}
+
+// Phase 1 with a segment table (SpanGroup::table_mode).  span_gather finds the row and the piece of every
+// destination vector and works out its source address lane by lane, some 150 vector instructions per 16 bytes.  Here
+// the (row, piece) pairs that touch the span - its SEGMENTS, at most one per lane - are worked out once, lane s
+// taking segment s, and left in LDS as 16-byte records; an item then needs one division for its row, a few compares
+// for its piece, one LDS read and an add.  That halves the kernel's vector and scalar instruction counts (counters);
+// its time on ragged rows stayed the same, since the wait for the gathered loads is what fills it.
+struct SpanSegment {   // 16 bytes in LDS
+  uint32_t d_lo, d_hi;  // (address of the piece row's first byte) - start, so that destination position y reads at d + y
+  uint32_t flags;       // 0: load; 1: the piece is a pad (zeros); 2: narrower than 16 bytes (gathered byte by byte)
+  int32_t end16;        // start + w - 16: the last position a 16-byte vector of this piece row may begin at
+};
+// The item of kind B a lane brings from span_table_build to span_table_gather (the first 16 bytes of its segment).
+template <class M>
+struct SpanRowStart {
+  typename M::cptr from;
+  uint32_t at;
+  bool on, zero;
+};
+
+struct SpanPieces4 {  // the first pieces of a member, read once by the wavefront (uniform)
+  SpanPiece c0, c1, c2, c3;
+};
+MMR_HD SpanPieces4 span_pieces4(const SpanPiece* pc, uint32_t k) {
+  return SpanPieces4{pc[0], pc[k > 1 ? 1 : 0], pc[k > 2 ? 2 : 0], pc[k > 3 ? 3 : 0]};
+}
+
+template <class M, class L, int LANES>
+MMR_HD SpanRowStart<M> span_table_build(const SpanGroup& g, const SpanMember& m, const SpanPieces4& pcs,
+                                        typename M::cptr safe, uint64_t x0, uint32_t len, uint32_t a, uint8_t* table,
+                                        uint32_t lane) {
+  const uint32_t W = g.W;
+  const uint64_t row0 = x0 < (1ull << 31) ? fdiv(static_cast<uint32_t>(x0), g.div_W) : x0 / W;
+  const uint32_t o0 = static_cast<uint32_t>(x0 - row0 * W);
+  const uint32_t nrows = fdiv(o0 + len + W - 1, g.div_W);
+  const uint32_t r0 = static_cast<uint32_t>(row0);
+  const uint32_t k = m.k;
+  const int32_t ilen = static_cast<int32_t>(len);
+  const bool on = lane < nrows * k;  // planner: nrows * k <= LANES in table mode
+  const uint32_t s = on ? lane : 0u;
+  const uint32_t rr = fdiv(s, m.div_k), p = s - rr * k;
+  SpanPick pk;
+  pk.take(true, pcs.c0);
+  if (k > 1) pk.take(p >= 1, pcs.c1);
+  if (k > 2) pk.take(p >= 2, pcs.c2);
+  if (k > 3) pk.take(p >= 3, pcs.c3);
+  const uint32_t row = r0 + rr;
+  const uint32_t r2 = fdiv(row, g.div_n1), r1 = row - r2 * g.n1;
+  const uint64_t src_row = pk.src + static_cast<uint64_t>(r2 * pk.s2 + r1 * pk.s1);
+  const int32_t start = static_cast<int32_t>(rr * W + pk.pcol) - static_cast<int32_t>(o0);
+  const bool wide = pk.w >= 16, fill = pk.src_slot == MMR_SLOT_FILL;
+  SpanSegment seg;
+  const uint64_t d = src_row - static_cast<uint64_t>(static_cast<int64_t>(start));
+  seg.d_lo = static_cast<uint32_t>(d);
+  seg.d_hi = static_cast<uint32_t>(d >> 32);
+  seg.flags = !wide ? 2u : (fill ? 1u : 0u);
+  seg.end16 = wide ? start + static_cast<int32_t>(pk.w) - 16 : -16;  // narrow: its vectors land in the spare bytes
+  if (on) L::store16u(table + (s << 4), V16{seg.d_lo, seg.d_hi, seg.flags, static_cast<uint32_t>(seg.end16)});
+  SpanRowStart<M> b;
+  b.on = on && wide;
+  b.zero = fill;
+  b.from = b.on && !fill ? reinterpret_cast<typename M::cptr>(src_row) : safe;
+  int32_t drel = start < -16 ? -16 : (start > ilen ? ilen : start);  // outside the span: into the spare bytes
+  b.at = static_cast<uint32_t>(static_cast<int32_t>(16 + a) + drel);
+  return b;
+}
+
+template <class M, class L, int LANES, int DEPTH>
+MMR_HD void span_table_gather(const SpanGroup& g, const SpanMember& m, const SpanPiece* pc, const SpanPieces4& pcs,
+                              typename M::cptr safe, uint64_t x0, uint32_t len, uint32_t a, uint8_t* lds,
+                              const uint8_t* table, const SpanRowStart<M>& b, uint32_t lane) {
+  const uint32_t W = g.W;
+  const uint64_t row0 = x0 < (1ull << 31) ? fdiv(static_cast<uint32_t>(x0), g.div_W) : x0 / W;
+  const uint32_t o0 = static_cast<uint32_t>(x0 - row0 * W);
+  const uint32_t k = m.k;
+  const uint32_t n_a = (len + a + 15) >> 4;  // aligned destination vectors that overlap the span
+  // one pass unless the span is a full one in a buffer that is not 16-byte aligned (one vector more than LANES * DEPTH)
+  for (uint32_t base = 0; base < n_a; base += LANES * DEPTH) {
+    V16 v[DEPTH + 1];
+    uint32_t at[DEPTH + 1];
+    bool live[DEPTH + 1], zero[DEPTH + 1];
+    typename M::cptr from[DEPTH + 1];
+#pragma unroll
+    for (int u = 0; u < DEPTH; ++u) {
+      const uint32_t i = base + lane + u * LANES;
+      live[u] = i < n_a;
+      const uint32_t v16 = i << 4;
+      const uint32_t y = !live[u] || v16 < a ? 0u : v16 - a;  // the vector's first byte inside the span
+      const uint32_t rr = fdiv(o0 + y, g.div_W), col = o0 + y - rr * W;
+      uint32_t p = 0;
+      if (k > 1) p += col >= pcs.c1.col ? 1u : 0u;
+      if (k > 2) p += col >= pcs.c2.col ? 1u : 0u;
+      if (k > 3) p += col >= pcs.c3.col ? 1u : 0u;
+      const V16 rec = L::load16(table + ((rr * k + p) << 4));
+      const int32_t end16 = static_cast<int32_t>(rec.w);
+      const int32_t yy = static_cast<int32_t>(y) < end16 ? static_cast<int32_t>(y) : end16;  // slides back to end with the piece
+      const uint64_t d = (static_cast<uint64_t>(rec.y) << 32) | rec.x;
+      zero[u] = rec.z != 0;
+      from[u] = live[u] && !zero[u] ? reinterpret_cast<typename M::cptr>(d + static_cast<uint64_t>(static_cast<int64_t>(yy))) : safe;
+      at[u] = static_cast<uint32_t>(static_cast<int32_t>(16 + a) + yy);
     }
+    live[DEPTH] = b.on && base == 0;
+    zero[DEPTH] = b.zero;
+    from[DEPTH] = base == 0 ? b.from : safe;
+    at[DEPTH] = b.at;
+#pragma unroll
+    for (int u = 0; u <= DEPTH; ++u) v[u] = M::load16u(from[u]);
+#pragma unroll
+    for (int u = 0; u <= DEPTH; ++u)
+      if (live[u]) L::store16u(lds + at[u], zero[u] ? V16{0, 0, 0, 0} : v[u]);
+  }
+  if (m.narrow) {
+    const uint32_t nrows = fdiv(o0 + len + W - 1, g.div_W);
+    span_gather_narrow<M, L, LANES>(g, pc, k, nrows, static_cast<uint32_t>(row0), o0, static_cast<int32_t>(len), a, lds, lane);
   }
 }
 

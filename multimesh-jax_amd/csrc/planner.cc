@@ -475,6 +475,8 @@ class Builder {
         }
         ps.m.k = static_cast<uint32_t>(ps.pieces.size());
         ps.m.wide = wide;
+        ps.m.narrow = ps.m.k - wide;
+        ps.m.div_k = make_fastdiv(std::max<uint32_t>(ps.m.k, 1));
         ps.m.div_wide = make_fastdiv(std::max<uint32_t>(wide, 1));
         spans.push_back(std::move(ps));
       });
@@ -765,7 +767,8 @@ void assemble_copies(std::vector<ProtoCopy>& protos, uint32_t order, int64_t fra
   plan->n_copy_chunks = next_chunk;
 }
 
-void assemble_spans(std::vector<ProtoSpan>& protos, uint32_t order, int64_t fraction_bytes, mmr_plan* plan) {
+void assemble_spans(std::vector<ProtoSpan>& protos, uint32_t order, int64_t fraction_bytes, bool segment_tables,
+                    mmr_plan* plan) {
   std::vector<size_t> at(protos.size());
   for (size_t i = 0; i < at.size(); ++i) at[i] = i;
   auto dst_key = [&](size_t i) { return std::make_tuple(protos[i].m.dst_slot, protos[i].m.dst, i); };
@@ -792,6 +795,11 @@ void assemble_spans(std::vector<ProtoSpan>& protos, uint32_t order, int64_t frac
     g.n_chunks = members * member_chunks;
     g.first_member = static_cast<uint32_t>(plan->span_members.size());
     g.il = make_interleave(members, member_chunks, fraction);
+    // few pieces per row and few (row, piece) pairs per span: the span kernel tabulates the pairs, one per lane
+    uint32_t most_pieces = 0;
+    for (size_t m = i; m < j; ++m) most_pieces = std::max(most_pieces, protos[at[m]].m.k);
+    const uint64_t rows_per_span = g.span / g.W + 2;
+    g.table_mode = segment_tables && most_pieces <= kSpanTablePieces && rows_per_span * most_pieces <= kSpanLanes ? 1 : 0;
     for (size_t m = i; m < j; ++m) {
       SpanMember mem = protos[at[m]].m;
       mem.first_piece = static_cast<uint32_t>(plan->span_pieces.size());
@@ -865,7 +873,8 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
   const uint32_t copy_order = options.order ? options.order : 2;
   const uint32_t span_order = options.order ? options.order : 4;
   assemble_copies(builder.copies, copy_order, (fraction_kib ? fraction_kib : 64) * 1024, plan);
-  assemble_spans(builder.spans, span_order, (fraction_kib ? fraction_kib : kDefaultSpanFractionKib) * 1024, plan);
+  assemble_spans(builder.spans, span_order, (fraction_kib ? fraction_kib : kDefaultSpanFractionKib) * 1024,
+                 (options.flags & MMR_PLAN_NO_SEGMENT_TABLES) == 0, plan);
   if (plan->n_copy_chunks > 0x7ff00000u || plan->n_span_chunks > 0x7ff00000u)
     return fail(MMR_INVALID_ARGUMENT, "plan of more than 2^31 chunks");
   const uint32_t order = options.order ? options.order : 2;

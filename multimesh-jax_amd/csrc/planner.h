@@ -36,7 +36,7 @@ struct mmr_plan {
 namespace mmr {
 
 constexpr uint32_t kDefaultChunkBytes = 8 * 1024;
-constexpr uint32_t kDefaultSpanBytes = 8 * 1024;      // destination bytes per workgroup of the span kernel
+constexpr uint32_t kDefaultSpanBytes = 4 * 1024;      // destination bytes per workgroup (one wavefront) of the span kernel
 constexpr int64_t kDefaultSpanFractionKib = 64;       // interleave round of the span groups, per tile
 constexpr int64_t kTransposeChunkBytes = 32 * 1024;  // a transpose chunk batches small tiles up to this many bytes
 

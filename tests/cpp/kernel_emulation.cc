@@ -265,22 +265,42 @@ int mmr_emulate_plan(const mmr_plan* plan, void* const* slot_ptrs, const size_t*
       const uint32_t a = static_cast<uint32_t>(m.dst + x0) & 15u;
       std::memset(lds, 0xA5 ^ static_cast<int>(ci & 0x3f), sizeof(lds));
       // a phase runs for every thread before the next one starts: the workgroup barrier
+      // shape 0 is the kernel's own launch shape; 1 runs the vector-by-vector gather on every group, also those the
+      // kernel uses a segment table for; 2 and 3 are other widths and depths of both
+      const mmr::SpanPiece* pc = pieces.data() + m.first_piece;
+      uint8_t* table = lds + mmr::kSpanStageBytes;
+      auto with_table = [&](auto lanes_c, auto depth_c) {
+        constexpr int LANES = decltype(lanes_c)::value, DEPTH = decltype(depth_c)::value;
+        const mmr::SpanPieces4 pcs = mmr::span_pieces4(pc, m.k);
+        std::vector<mmr::SpanRowStart<HostMem>> starts(LANES);
+        for (uint32_t tid = 0; tid < LANES; ++tid)
+          starts[tid] = mmr::span_table_build<HostMem, HostLds, LANES>(g, m, pcs, safe, x0, len, a, table, tid);
+        for (uint32_t tid = 0; tid < LANES; ++tid)
+          mmr::span_table_gather<HostMem, HostLds, LANES, DEPTH>(g, m, pc, pcs, safe, x0, len, a, lds, table, starts[tid], tid);
+        for (uint32_t tid = 0; tid < LANES; ++tid) mmr::span_write<HostMem, HostLds, LANES, DEPTH>(dst, len, a, lds, tid);
+      };
+      auto without = [&](auto threads_c, auto unroll_c) {
+        constexpr int THREADS = decltype(threads_c)::value, UNROLL = decltype(unroll_c)::value;
+        for (uint32_t tid = 0; tid < THREADS; ++tid)
+          mmr::span_gather<HostMem, HostLds, THREADS, UNROLL>(g, m, pieces.data(), safe, x0, len, a, lds, tid);
+        for (uint32_t tid = 0; tid < THREADS; ++tid) mmr::span_write<HostMem, HostLds, THREADS, UNROLL>(dst, len, a, lds, tid);
+      };
+      using std::integral_constant;
       switch (shape) {
         case 1:
-          for (uint32_t tid = 0; tid < 128; ++tid) mmr::span_gather<HostMem, HostLds, 128, 4>(g, m, pieces.data(), safe, x0, len, a, lds, tid);
-          for (uint32_t tid = 0; tid < 128; ++tid) mmr::span_write<HostMem, HostLds, 128, 4>(dst, len, a, lds, tid);
+          without(integral_constant<int, 128>{}, integral_constant<int, 4>{});
           break;
         case 2:
-          for (uint32_t tid = 0; tid < 256; ++tid) mmr::span_gather<HostMem, HostLds, 256, 1>(g, m, pieces.data(), safe, x0, len, a, lds, tid);
-          for (uint32_t tid = 0; tid < 256; ++tid) mmr::span_write<HostMem, HostLds, 256, 1>(dst, len, a, lds, tid);
+          if (g.table_mode) with_table(integral_constant<int, 64>{}, integral_constant<int, 5>{});
+          else without(integral_constant<int, 256>{}, integral_constant<int, 1>{});
           break;
         case 3:
-          for (uint32_t tid = 0; tid < 512; ++tid) mmr::span_gather<HostMem, HostLds, 512, 3>(g, m, pieces.data(), safe, x0, len, a, lds, tid);
-          for (uint32_t tid = 0; tid < 512; ++tid) mmr::span_write<HostMem, HostLds, 512, 3>(dst, len, a, lds, tid);
+          if (g.table_mode) with_table(integral_constant<int, 64>{}, integral_constant<int, 8>{});
+          else without(integral_constant<int, 32>{}, integral_constant<int, 3>{});
           break;
         default:
-          for (uint32_t tid = 0; tid < 256; ++tid) mmr::span_gather<HostMem, HostLds, 256, 2>(g, m, pieces.data(), safe, x0, len, a, lds, tid);
-          for (uint32_t tid = 0; tid < 256; ++tid) mmr::span_write<HostMem, HostLds, 256, 2>(dst, len, a, lds, tid);
+          if (g.table_mode) with_table(integral_constant<int, mmr::kSpanLanes>{}, integral_constant<int, mmr::kSpanDepth>{});
+          else without(integral_constant<int, mmr::kSpanLanes>{}, integral_constant<int, mmr::kSpanDepth>{});
           break;
       }
     });

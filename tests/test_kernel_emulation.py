@@ -94,6 +94,33 @@ def test_ragged_rows_through_the_kernel_code(a, chunk_bytes, shape):
     _check([a], [g], chunk_bytes=chunk_bytes, shape=shape)
 
 
+@st.composite
+def ragged_3d(draw):
+    """Long ragged rows under two row dims: the span kernel walks them piece row by piece row, across the boundary
+    between the inner and the outer row dim and, with the first dim split on one side only, across tiles."""
+    outer, inner = draw(st.integers(1, 5)), draw(st.integers(1, 7))
+    cols = draw(st.integers(130, 2600))
+    type_ = draw(st.sampled_from(["U8", "BF16"]))
+    st_src, st_dst = draw(st.integers(1, 4)), draw(st.integers(1, 5))
+    od = draw(st.integers(1, 2))
+    return {"name": "rag3", "type": type_, "shape": (outer, inner, cols),
+            "src": {"dims": [(outer, 1, 0), (inner, 1, 1), (cols, st_src, 2)], "dev_start": 0, "dev_count": st_src},
+            "dst": {"dims": [(outer, od, 1), (inner, 1, 2), (cols, st_dst, 0)], "dev_start": 20,
+                    "dev_count": od * st_dst},
+            "seed": 0, "dist": "raw"}
+
+
+@given(ragged_3d(), st.sampled_from([0, 512, 4096]), st.sampled_from([0, 1, 2, 3]))
+@settings(max_examples=120, deadline=None)
+def test_long_ragged_rows_under_two_row_dims(a, chunk_bytes, shape):
+    from oracle import reshard_oracle as ro
+    item = ro.ITEMSIZE[a["type"]]
+    rng = np.random.Generator(np.random.PCG64(29))
+    g = rng.integers(0, 256, size=int(np.prod(a["shape"])) * item, dtype=np.uint8).view(
+        ro.raw_dtype(a["type"])).reshape(a["shape"])
+    _check([a], [g], chunk_bytes=chunk_bytes, shape=shape)
+
+
 @pytest.mark.parametrize("type_", ["U8", "BF16", "F32", "F64", "C128"])
 @pytest.mark.parametrize("shape", [(256, 384), (192, 200), (130, 256)])
 def test_transposed_layout_vector_and_element_tiles(type_, shape):

@@ -207,8 +207,8 @@ def test_ragged_rows_become_destination_spans():
     s = plan.stats
     assert s["n_copy16_chunks"] == 0 and s["n_copy_generic_chunks"] == 0 and s["n_transpose_chunks"] == 0
     assert s["n_groups"] == 2  # one per array, five interleaved tiles each
-    # destination shards of 8 x 3280 and 11008 x 820 bytes, five each, in spans of 8 KiB
-    assert s["n_span_chunks"] == 5 * (-(-8 * 3280 // 8192)) + 5 * (-(-11008 * 820 // 8192))
+    # destination shards of 8 x 3280 and 11008 x 820 bytes, five each, in spans of 4 KiB
+    assert s["n_span_chunks"] == 5 * (-(-8 * 3280 // 4096)) + 5 * (-(-11008 * 820 // 4096))
     assert s["table_bytes"] < 4096
     pieces = plan.copy_chunks(2)
     fp8 = pieces[pieces["d1"] == 820]
