@@ -260,7 +260,8 @@ def record_traffic(args):
         with open(files[0]) as f:
             for row in csv.DictReader(f):
                 if "mmr_" in row["Kernel_Name"] and row["Counter_Name"] == counter:
-                    per_kernel.setdefault(row["Kernel_Name"].split("(")[0], []).append(float(row["Counter_Value"]))
+                    name = row["Kernel_Name"].replace("(anonymous namespace)::", "").replace("void ", "")
+                    per_kernel.setdefault(name.split("(")[0], []).append(float(row["Counter_Value"]))
         name, values = max(per_kernel.items(), key=lambda kv: sum(kv[1]))
         kernel = name
         out[counter] = {"kib_mean": sum(values) / len(values), "kib_min": min(values), "kib_max": max(values),
