@@ -213,16 +213,14 @@ typedef struct {
 
 typedef struct {
   uint32_t chunk_bytes; /* target bytes per copy chunk, 0 = default */
-  uint32_t order;       /* 0 = default (2 for aligned chunks and tiles, 4 for ragged chunks); 1 generation order,
+  uint32_t order;       /* 0 = default (2 for copy groups and tiles, 4 for span groups); 1 generation order,
                            2 by destination address, 3 by source address, 4 = by destination with the tiles of an
                            array interleaved in equal fractions (the same rows of all tiles together) */
   uint32_t xcd_mode;    /* workgroup -> chunk mapping. 0 = default; 1 = chunk i is workgroup i (the hardware deals
                            consecutive workgroups round-robin over the 8 XCDs); 2 = each XCD takes a contiguous
                            eighth of the table; G >= 16 = runs of G table neighbours share an XCD (and its L2) */
-  uint32_t flags;       /* MMR_PLAN_ALL_GENERIC: route aligned chunks through the generic kernel too (testing);
-                           MMR_PLAN_NO_AUTOTUNE: keep the default table order instead of timing a few orders on
-                           the first reshard of a descriptor pair (only done when `order` is 0);
-                           bits 8-23: KiB per tile and fraction for order 4 (0 = default, 64) */
+  uint32_t flags;       /* MMR_PLAN_* bits above (testing and probing switches);
+                           bits 8-23: KiB per tile and round for order 4 (0 = default, 64) */
 } mmr_plan_options;
 
 typedef struct {
