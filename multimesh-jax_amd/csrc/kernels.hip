@@ -94,13 +94,9 @@ __device__ __forceinline__ gchar* slot_base(void* const* __restrict__ ptrs, uint
   return (gchar*)(static_cast<char*>(ptrs[slot])) + off;
 }
 
-// Launch shape of the aligned kernel (overridable at build time for tuning runs).
-#ifndef MMR_COPY16_UNROLL
-#define MMR_COPY16_UNROLL 2
-#endif
-#ifndef MMR_COPY16_NT_LOADS
-#define MMR_COPY16_NT_LOADS true
-#endif
+// Launch shape of the aligned kernel: 256 threads, 2 vectors each (8 KiB per workgroup), nontemporal both ways.
+constexpr int kCopy16Unroll = 2;
+constexpr bool kCopy16NtLoads = true;
 
 // Copy groups: the workgroup works its chunk out from the group table (bound: absolute addresses).  `groups` and
 // `pieces` are wave-uniform reads (scalar loads); the records are taken by value so that their loads leave together.
@@ -113,7 +109,7 @@ __device__ __forceinline__ void copy_group_chunk(const CopyGroup* __restrict__ g
   const mmr_copy_chunk c = copy_chunk_of(g, p, d);
   gchar* dst = (gchar*)(c.dst_off);
   gcchar* src = c.src_slot == MMR_SLOT_FILL ? dst : (gcchar*)(c.src_off);  // never read when filling
-  copy_group_rows<DeviceMem<MMR_COPY16_NT_LOADS, true>, THREADS, UNROLL>(g, p, c, src, dst, threadIdx.x);
+  copy_group_rows<DeviceMem<kCopy16NtLoads, true>, THREADS, UNROLL>(g, p, c, src, dst, threadIdx.x);
 }
 
 // DIRECT: the table has at most kMaxDirectGroups groups and `starts` holds their first chunks (no hint lookup).
@@ -201,19 +197,10 @@ __global__ __launch_bounds__(THREADS) void mmr_copy_generic_kernel(const mmr_cop
   generic_chunk<DeviceMem<NTL, NTS>, THREADS, UNROLL>(c, src, dst, threadIdx.x);
 }
 
-// Launch shape of the generic kernel (overridable at build time for tuning runs).
-#ifndef MMR_GENERIC_THREADS
-#define MMR_GENERIC_THREADS 256
-#endif
-#ifndef MMR_GENERIC_UNROLL
-#define MMR_GENERIC_UNROLL 2
-#endif
-#ifndef MMR_GENERIC_NT_LOADS
-#define MMR_GENERIC_NT_LOADS false
-#endif
-constexpr int kGenericThreads = MMR_GENERIC_THREADS;
-constexpr int kGenericUnroll = MMR_GENERIC_UNROLL;
-constexpr bool kGenericNtLoads = MMR_GENERIC_NT_LOADS;
+// Launch shape of the generic kernel; cacheable loads (a source line shared by two chunks is fetched once).
+constexpr int kGenericThreads = 256;
+constexpr int kGenericUnroll = 2;
+constexpr bool kGenericNtLoads = false;
 
 // Orders the LDS accesses of the lanes of one wave: what a lane wrote before is visible to the others after.
 __device__ __forceinline__ void wave_sync() {
@@ -384,10 +371,10 @@ hipError_t launch_copy_groups(const CopyGroup* d_groups, uint32_t n_groups, cons
   GroupStarts s;
   for (uint32_t i = 0; i < kMaxDirectGroups; ++i) s.first[i] = starts && i < n_groups ? starts[i] : 0xffffffffu;
   if (starts && n_groups <= kMaxDirectGroups)
-    hipLaunchKernelGGL((mmr_copy16_kernel<256, MMR_COPY16_UNROLL, true>), dim3(grid_size(n, group)), dim3(256), 0, stream,
+    hipLaunchKernelGGL((mmr_copy16_kernel<256, kCopy16Unroll, true>), dim3(grid_size(n, group)), dim3(256), 0, stream,
                        d_groups, n_groups, d_pieces, d_hints, static_cast<uint32_t>(n), group, s);
   else
-    hipLaunchKernelGGL((mmr_copy16_kernel<256, MMR_COPY16_UNROLL, false>), dim3(grid_size(n, group)), dim3(256), 0, stream,
+    hipLaunchKernelGGL((mmr_copy16_kernel<256, kCopy16Unroll, false>), dim3(grid_size(n, group)), dim3(256), 0, stream,
                        d_groups, n_groups, d_pieces, d_hints, static_cast<uint32_t>(n), group, s);
   return hipGetLastError();
 }
@@ -398,7 +385,7 @@ hipError_t launch_copy_groups_inline(const InlineCopyTable& table, uint32_t xcd_
   if (hipError_t e = check_grid(n)) return e;
   if (table.n_groups > kInlineCopyGroups) return hipErrorInvalidValue;
   const uint32_t group = xcd_group_of(n, xcd_mode);
-  hipLaunchKernelGGL((mmr_copy16_inline_kernel<256, MMR_COPY16_UNROLL>), dim3(grid_size(n, group)), dim3(256), 0, stream,
+  hipLaunchKernelGGL((mmr_copy16_inline_kernel<256, kCopy16Unroll>), dim3(grid_size(n, group)), dim3(256), 0, stream,
                      table, group);
   return hipGetLastError();
 }

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 import multimesh_jax_amd as mm
-from multimesh_jax_amd import workloads
+from multimesh_jax_amd import _binding as B, workloads
 from oracle import reshard_cpu, reshard_oracle as ro
 
 from helpers import lib_shape, oracle_outputs, oracle_shape, raw_global
@@ -45,6 +45,28 @@ def test_benchmark_config_full_size(ctx, index):
     gs = [workloads.generate(a) for a in arrays]
     outs = gpu_reshard(ctx, arrays, gs)
     _compare(arrays, gs, outs)
+
+
+@pytest.mark.parametrize("flags", [0, B.MMR_PLAN_NO_SEGMENT_TABLES, B.MMR_PLAN_NO_SPAN, B.MMR_PLAN_ALL_GENERIC,
+                                   B.MMR_PLAN_ALL_GENERIC | B.MMR_PLAN_NO_SEGMENT_TABLES])
+def test_ragged_rows_through_every_gather(ctx, flags):
+    """Ragged rows through the span kernel with and without its segment table, through the generic kernel, and aligned
+    configurations forced through both span gathers: the same bytes every way."""
+    say("ragged rows, plan flags %d" % flags)
+    ctx.set_plan_options(0, 0, 0, flags)
+    try:
+        cases = [workloads.config(5), workloads.config(6, 4), workloads.config(2, 8), workloads.config(3, 4)]
+        # long ragged rows under two row dims, 1 to 6 pieces per destination row
+        for cols, s_src, s_dst in ((1031, 3, 2), (2600, 4, 5), (700, 6, 1), (130, 1, 5)):
+            cases.append([{"name": "rag3", "type": "U8", "shape": (3, 50, cols),
+                           "src": {"dims": [(3, 1, 0), (50, 1, 1), (cols, s_src, 2)], "dev_start": 0, "dev_count": s_src},
+                           "dst": {"dims": [(3, 1, 1), (50, 1, 2), (cols, s_dst, 0)], "dev_start": 9, "dev_count": s_dst},
+                           "seed": cols, "dist": "raw"}])
+        for arrays in cases:
+            gs = [workloads.generate(a) for a in arrays]
+            _compare(arrays, gs, gpu_reshard(ctx, arrays, gs))
+    finally:
+        ctx.set_plan_options(0, 0)
 
 
 @pytest.mark.parametrize("chunk_bytes,order", [(4096, 1), (16384, 3), (262144, 2)])
