@@ -314,14 +314,18 @@ MMR_HD void generic_chunk(const mmr_copy_chunk& c, typename M::cptr src, typenam
 template <int ITEM>
 struct TransposeTile {
   // wave sub-tile: 128 bytes (or more) wide on both sides, so every access of 8 lanes is a full 128-byte line
-  static constexpr int kEX = ITEM == 1 ? 128 : (ITEM == 2 ? 64 : 32);
-  static constexpr int kEY = ITEM == 1 ? 128 : (ITEM == 16 ? 16 : (ITEM == 8 ? 32 : 64));
+  static constexpr int kEX = ITEM == 1 ? 128 : (ITEM == 2 || ITEM == 4 ? 64 : 32);
+  static constexpr int kEY = ITEM == 1 || ITEM == 4 ? 128 : (ITEM == 16 ? 16 : (ITEM == 8 ? 32 : 64));
   // Sub-tiles per workgroup tile, and the threads that share one.  1-byte elements: the smallest sub-tile is
   // already 16 KiB, too many registers for one wave, so the four waves of the workgroup share a single sub-tile
-  // (and synchronise with a workgroup barrier instead of a wave fence).
-  static constexpr int kWX = ITEM == 1 ? 1 : 2, kWY = kWX;
+  // (and synchronise with a workgroup barrier instead of a wave fence).  4-byte elements: the four waves share the
+  // whole 64 x 128 tile too, whose rows are 256 and 512 bytes long, and 16 lanes take a 256-byte piece of a row
+  // (measured 1.6 % faster than four 32 x 64 sub-tiles with 128-byte pieces; for 2-byte elements the same change
+  // measured 0.5 % slower and was not made).
+  static constexpr bool kShared = ITEM == 1 || ITEM == 4;
+  static constexpr int kWX = kShared ? 1 : 2, kWY = kWX;
   static constexpr int kWaves = kWX * kWY;                   // number of sub-tiles
-  static constexpr int kGroupThreads = ITEM == 1 ? 256 : 64; // threads per sub-tile
+  static constexpr int kGroupThreads = kShared ? 256 : 64;   // threads per sub-tile
   static constexpr int kThreads = kGroupThreads * kWaves;
   static constexpr int kTileX = kEX * kWX, kTileY = kEY * kWY;
   static constexpr int kVec = 16 / ITEM;                     // elements per 16-byte vector
@@ -329,6 +333,8 @@ struct TransposeTile {
   static constexpr int kRowBytes = kEY * ITEM;               // bytes per LDS row (no padding)
   static constexpr int kSrcVecs = kEX / kVec;                // 16-byte groups per source row of a sub-tile
   static constexpr int kDstVecs = kEY / kVec;                // 16-byte groups per destination row of a sub-tile
+  static constexpr int kSrcSeg = ITEM == 4 ? 16 : 8;         // lanes that share a row segment when loading ...
+  static constexpr int kDstSeg = ITEM == 4 ? 16 : 8;         // ... and when storing (transpose_task)
   static constexpr int kRowPacks = kEY / kPack;              // packed source-row groups per sub-tile
   static constexpr int kWaveLdsBytes = kEX * kEY * ITEM;     // one sub-tile's slice
   static constexpr int kLdsBytes = kWaveLdsBytes * kWaves;
@@ -388,13 +394,14 @@ MMR_HD T element_of(const V16& v, int i) {
   }
 }
 
-// Task t of a wave's phase -> (row index, 16-byte group within the row).  8
-// consecutive lanes take the 8 groups of one 128-byte row segment, the next 8
-// lanes the same segment of the next row; rows wider than 128 bytes are covered
-// segment after segment.  `rows` is the number of rows in the phase.
-MMR_HD void transpose_task(uint32_t t, uint32_t rows, uint32_t* row, uint32_t* group) {
-  const uint32_t r = t >> 3;
-  *group = (t & 7u) + ((r / rows) << 3);
+// Task t of a wave's phase -> (row index, 16-byte group within the row).  `seg`
+// consecutive lanes take the groups of one row segment of seg * 16 bytes (8:
+// a 128-byte line; 16: two), the next `seg` lanes the same segment of the next
+// row; wider rows are covered segment after segment.  `rows` is the number of
+// rows in the phase.
+MMR_HD void transpose_task(uint32_t t, uint32_t rows, uint32_t* row, uint32_t* group, uint32_t seg) {
+  const uint32_t r = t / seg;
+  *group = (t % seg) + (r / rows) * seg;
   *row = r % rows;
 }
 
@@ -468,7 +475,7 @@ MMR_HD void transpose_load_vec(const mmr_transpose_chunk& c, typename M::cptr sr
 #pragma unroll
   for (int k = 0; k < kTasks; ++k) {
     uint32_t yg, xv;
-    transpose_task(lane + k * G::kGroupThreads, G::kRowPacks, &yg, &xv);
+    transpose_task(lane + k * G::kGroupThreads, G::kRowPacks, &yg, &xv, G::kSrcSeg);
     const bool inside = y0 + yg * G::kPack < c.ny && x0 + xv * G::kVec < c.nx;
     const uint32_t yl = inside ? yg * G::kPack : 0u, xl = inside ? xv : 0u;
 #pragma unroll
@@ -478,7 +485,7 @@ MMR_HD void transpose_load_vec(const mmr_transpose_chunk& c, typename M::cptr sr
 #pragma unroll
   for (int k = 0; k < kTasks; ++k) {
     uint32_t yg, xv;
-    transpose_task(lane + k * G::kGroupThreads, G::kRowPacks, &yg, &xv);
+    transpose_task(lane + k * G::kGroupThreads, G::kRowPacks, &yg, &xv, G::kSrcSeg);
     const uint32_t ybyte = yg * G::kPack * static_cast<uint32_t>(sizeof(T));  // byte of y within LDS row x
 #pragma unroll
     for (int i = 0; i < G::kVec; ++i) {
@@ -511,14 +518,14 @@ MMR_HD void transpose_store_vec(const mmr_transpose_chunk& c, typename M::ptr ds
 #pragma unroll
   for (int k = 0; k < kTasks; ++k) {
     uint32_t x, yv;
-    transpose_task(lane + k * G::kGroupThreads, G::kEX, &x, &yv);
+    transpose_task(lane + k * G::kGroupThreads, G::kEX, &x, &yv, G::kDstSeg);
     if (x0 + x < c.nx && y0 + yv * G::kVec < c.ny)
       v[k] = *reinterpret_cast<const V16*>(tile + x * G::kRowBytes + ((yv ^ transpose_swizzle<sizeof(T)>(x)) << 4));
   }
 #pragma unroll
   for (int k = 0; k < kTasks; ++k) {
     uint32_t x, yv;
-    transpose_task(lane + k * G::kGroupThreads, G::kEX, &x, &yv);
+    transpose_task(lane + k * G::kGroupThreads, G::kEX, &x, &yv, G::kDstSeg);
     if (x0 + x < c.nx && y0 + yv * G::kVec < c.ny) M::store16(d + (x * c.dst_xstride + static_cast<int64_t>(yv) * 16), v[k]);
   }
 }
@@ -540,7 +547,7 @@ MMR_HD void transpose_load_general(const mmr_transpose_chunk& c, typename M::cpt
 #pragma unroll
   for (int k = 0; k < kTasks; ++k) {
     uint32_t yg, xv;
-    transpose_task(lane + k * G::kGroupThreads, G::kRowPacks, &yg, &xv);
+    transpose_task(lane + k * G::kGroupThreads, G::kRowPacks, &yg, &xv, G::kSrcSeg);
     xs[k] = xv * G::kVec + G::kVec > snx ? snx - G::kVec : xv * G::kVec;  // slides inwards, overlapping its neighbour
 #pragma unroll
     for (int p = 0; p < G::kPack; ++p) {
@@ -551,7 +558,7 @@ MMR_HD void transpose_load_general(const mmr_transpose_chunk& c, typename M::cpt
 #pragma unroll
   for (int k = 0; k < kTasks; ++k) {
     uint32_t yg, xv;
-    transpose_task(lane + k * G::kGroupThreads, G::kRowPacks, &yg, &xv);
+    transpose_task(lane + k * G::kGroupThreads, G::kRowPacks, &yg, &xv, G::kSrcSeg);
 #pragma unroll
     for (int i = 0; i < G::kVec; ++i) {
       uint8_t* at = tile + transpose_lds_offset<sizeof(T)>(xs[k] + i, yg * G::kPack);
@@ -582,7 +589,7 @@ MMR_HD void transpose_store_general(const mmr_transpose_chunk& c, typename M::pt
 #pragma unroll
   for (int k = 0; k < kTasks; ++k) {
     uint32_t x, yv;
-    transpose_task(lane + k * G::kGroupThreads, G::kEX, &x, &yv);
+    transpose_task(lane + k * G::kGroupThreads, G::kEX, &x, &yv, G::kDstSeg);
     ys[k] = yv * G::kVec;
     if (x < snx && ys[k] < sny) {
       if (ys[k] + G::kVec <= sny) {
@@ -599,7 +606,7 @@ MMR_HD void transpose_store_general(const mmr_transpose_chunk& c, typename M::pt
 #pragma unroll
   for (int k = 0; k < kTasks; ++k) {
     uint32_t x, yv;
-    transpose_task(lane + k * G::kGroupThreads, G::kEX, &x, &yv);
+    transpose_task(lane + k * G::kGroupThreads, G::kEX, &x, &yv, G::kDstSeg);
     if (x < snx && yv * G::kVec < sny)
       M::template storeu<V16>(d + (x * c.dst_xstride + static_cast<int64_t>(ys[k]) * static_cast<int64_t>(sizeof(T))), v[k]);
   }

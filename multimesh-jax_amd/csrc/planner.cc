@@ -886,15 +886,21 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
       });
     };
     sort_generic(plan->generic);
-    // Tiles: by destination in blocks of 8 x 8 tiles rather than row after row, so the workgroups in flight
-    // together cover a compact region with long contiguous pieces on the source side as well as on the
-    // destination side (measured +10 % over plain destination order).
+    // Tiles: in blocks of 8 x 8 tiles (long contiguous pieces on the source side as well as on the destination
+    // side: +10 % over plain destination order), the blocks taken diagonal after diagonal - (block column + block
+    // row + 3 * destination buffer) mod 8 - rather than column after column: the tiles in flight together then differ
+    // in their source rows as well as in their destination rows.  With power-of-two pitches, rows one tile apart lie
+    // a multiple of the memory channels' interleave apart, and a launch that walks one side in address order keeps
+    // hitting the same few channels on the other side (measured +3 to +12 % on power-of-two transposes of 1-, 2- and
+    // 4-byte elements in six shapes and splits, -3 % on a 6144 x 6144 one; other block shapes, moduli and key orders
+    // won on some of them and lost more on others).
     auto tile_key = [](const mmr_transpose_chunk& c) {
       const uint64_t pitch = c.dst_xstride > 0 ? static_cast<uint64_t>(c.dst_xstride) : 1;
       uint32_t tx = 0, ty = 0;
       transpose_tile_extent(c.itemsize, &tx, &ty);
       const uint64_t x = c.dst_off / pitch, y = c.dst_off % pitch;  // destination row, byte within it
-      return std::make_tuple(c.dst_slot, x / (8ull * tx), y / (8ull * ty * c.itemsize), x, y);
+      const uint64_t bx = x / (8ull * tx), by = y / (8ull * ty * c.itemsize);
+      return std::make_tuple((bx + by + 3ull * c.dst_slot) % 8ull, bx, c.dst_slot, x, y);
     };
     std::stable_sort(plan->transposes.begin(), plan->transposes.end(),
                      [&](const mmr_transpose_chunk& a, const mmr_transpose_chunk& b) {
