@@ -91,7 +91,6 @@ def cpu_baseline(arrays, gs, seconds=12.0):
                       % (reps, dt, threads, visible, reps1, dt1)}, out
 
 
-NO_PARITY = False  # --no-parity: probing builds whose kernels move the wrong bytes on purpose
 
 
 def percentile(sorted_values, q):
@@ -107,8 +106,6 @@ def check_parity(ctx, arrays, gs, dsts, sample_only):
     from gpu_helpers import read_all
     from helpers import oracle_outputs
 
-    if NO_PARITY:
-        return 0
     picked = range(len(arrays))
     if sample_only:
         picked = [i for i, a in enumerate(arrays) if a["name"].startswith("layer00.") or "." not in a["name"]]
@@ -315,7 +312,6 @@ def main():
     ap.add_argument("--order", type=int, default=0)
     ap.add_argument("--xcd-mode", type=int, default=0)
     ap.add_argument("--flags", type=int, default=0)
-    ap.add_argument("--no-parity", action="store_true", help="skip the comparison with the oracle (probing builds only)")
     ap.add_argument("--name", type=str, default="", help="only the arrays whose name contains this")
     ap.add_argument("--scale", type=int, default=1, help="divide the large extents (probing only)")
     ap.add_argument("--workload-json", type=str, default="",
@@ -328,8 +324,6 @@ def main():
     if args.record_traffic:
         record_traffic(args)
         return
-    global NO_PARITY
-    NO_PARITY = args.no_parity
 
     import multimesh_jax_amd as mm
     from multimesh_jax_amd import workloads
