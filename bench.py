@@ -379,6 +379,9 @@ def main():
             "median_ms": round(res["median_ms"], 5), "p10_ms": round(res["p10_ms"], 5), "p90_ms": round(res["p90_ms"], 5),
             "launches_timed_one_by_one": res["laps"], "median_GB/s": round(res["median_gbs"], 1),
             "launches_per_step": res["launches"],
+            # the same launch priced at the bytes the HBM counters saw instead of the algorithmic ones
+            "traffic_over_algorithmic": round(traffic / res["alg_bytes"], 4) if traffic else None,
+            "counter_GB/s": round(traffic / (res["kernel_ms"] * 1e-3) / 1e9, 1) if traffic else None,
         },
     }
     if not args.no_cpu_baseline and args.config == 2 and args.scale == 1 and not args.workload_json:

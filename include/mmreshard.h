@@ -239,7 +239,7 @@ typedef struct {
   int64_t n_slots;
   int64_t order_used;          /* table order in effect: 0 = the default mix, else a value of mmr_plan_options.order */
   int64_t interleave_kib;      /* order 4 only: KiB per tile and fraction */
-  int64_t orders_timed;        /* how many table orders the first reshard timed (0 = no tuning) */
+  int64_t orders_timed;        /* how many launch orders mmr_reshard_tune timed for this plan (0 = never tuned) */
 } mmr_plan_stats;
 
 int mmr_plan_create(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int32_t n_arrays,

@@ -16,8 +16,8 @@
 //   * span groups - ragged rows.  The destination tile is dense, so a chunk is
 //     a SPAN of destination bytes cut at multiples of the span size counted from
 //     the buffer's base: the workgroup gathers the pieces of every row that
-//     touches the span into LDS, laid out as the destination is (aligned 16-byte
-//     global loads, unaligned LDS writes), and then writes the span out as whole
+//     touches the span into LDS, laid out as the destination is (16-byte global
+//     loads and LDS writes at any byte alignment), and then writes the span out as whole
 //     aligned 16-byte vectors - no partial line ever reaches memory from the
 //     middle of a tile.
 // The same code runs on the GPU (kernels.hip) and, with a bounds-checking

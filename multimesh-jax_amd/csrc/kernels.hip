@@ -328,11 +328,11 @@ hipError_t check_grid(int64_t n) { return (n < 0 || n > 0x7ff00000LL) ? hipError
 
 }  // namespace
 
-// Launch shapes are the measured optimum on MI355X for 8 KiB (aligned) and
-// 7 KiB (generic) chunks: 256 threads, up to 8 (aligned) or 2 (generic) 16-byte
-// accesses in flight per lane before the first store; one workgroup per chunk
-// (persistent workgroups that loop over the table, 4 to 16 per CU, with the
-// next chunk record prefetched, were 2-18 % slower on every configuration).
+// Launch shapes are the measured optimum on MI355X: 256 threads and 2 16-byte
+// accesses in flight per lane for 8 KiB (aligned) and 7 KiB (generic) chunks,
+// one wavefront and 4 + 1 accesses per lane for 4 KiB spans; one workgroup per
+// chunk (persistent workgroups that loop over the table, 4 to 16 per CU, with
+// the next chunk record prefetched, were 2-18 % slower on every configuration).
 hipError_t static_scratch_address(int device, void** out) {
   constexpr int kMaxDevices = 64;
   static std::mutex mu;
