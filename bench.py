@@ -180,6 +180,14 @@ def measure(ctx, mm, workloads, args, config):
     ctx.Sync()
     wall_s = time.perf_counter() - t0
     syncs_in_region = ctx.stats["host_blocking_syncs"] - syncs_before
+    # the same bracket five more times over 50 back-to-back launches each: the median of the five means
+    brackets = []
+    for _ in range(5):
+        ctx.StartTimer()
+        for i in range(50):
+            step(i)
+        brackets.append(ctx.StopTimer() / 50)
+    brackets.sort()
     # per-launch distribution: a timing mark between each two of at least 50 back-to-back launches
     n_laps = max(50, min(args.steps, 500))
     ctx.Lap()
@@ -212,6 +220,7 @@ def measure(ctx, mm, workloads, args, config):
         "kernel_ms": kernel_ms / args.steps,
         "achieved": alg_bytes / (kernel_ms / args.steps * 1e-3) / 1e9,
         "median_ms": med, "p10_ms": percentile(laps, 0.1), "p90_ms": percentile(laps, 0.9), "laps": len(laps),
+        "bracket_median_ms": brackets[2], "bracket_min_ms": brackets[0], "bracket_max_ms": brackets[-1],
         "median_gbs": alg_bytes / (med * 1e-3) / 1e9 if med else None,
         "launches": launches, "plan": plan, "plan_build_ms": plan_build_ms, "plan_table_bytes": table_bytes,
         "kernel": kernel, "n_arrays": len(arrays), "sets": len(sets), "order_used": order_used,
@@ -280,6 +289,7 @@ def summary(r):
     return {"GB/s": round(r["achieved"], 1), "frac_hbm_peak": round(r["achieved"] / HBM_PEAK_GBS, 4),
             "kernel_ms": round(r["kernel_ms"], 5), "median_ms": round(r["median_ms"], 5),
             "p10_ms": round(r["p10_ms"], 5), "p90_ms": round(r["p90_ms"], 5), "launches_timed": r["laps"],
+            "bracket_median_ms": round(r["bracket_median_ms"], 5),
             "median_GB/s": round(r["median_gbs"], 1), "algorithmic_bytes": r["alg_bytes"],
             "launches_per_step": r["launches"], "kernel": r["kernel"], "buffer_sets": r["sets"],
             "plan_build_ms_cold": round(r["plan_build_ms"], 3), "plan_table_bytes": r["plan_table_bytes"],
@@ -378,6 +388,9 @@ def main():
             "kernel": res["kernel"], "kernel_ms": round(res["kernel_ms"], 5),
             "median_ms": round(res["median_ms"], 5), "p10_ms": round(res["p10_ms"], 5), "p90_ms": round(res["p90_ms"], 5),
             "launches_timed_one_by_one": res["laps"], "median_GB/s": round(res["median_gbs"], 1),
+            # median (min, max) of five brackets of 50 back-to-back launches each, events on the library's stream
+            "bracket_median_ms": round(res["bracket_median_ms"], 5), "bracket_min_ms": round(res["bracket_min_ms"], 5),
+            "bracket_max_ms": round(res["bracket_max_ms"], 5),
             "launches_per_step": res["launches"],
             # the same launch priced at the bytes the HBM counters saw instead of the algorithmic ones
             "traffic_over_algorithmic": round(traffic / res["alg_bytes"], 4) if traffic else None,
