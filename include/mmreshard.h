@@ -220,7 +220,7 @@ typedef struct {
                            consecutive workgroups round-robin over the 8 XCDs); 2 = each XCD takes a contiguous
                            eighth of the table; G >= 16 = runs of G table neighbours share an XCD (and its L2) */
   uint32_t flags;       /* MMR_PLAN_* bits above (testing and probing switches);
-                           bits 8-23: KiB per tile and round for order 4 (0 = default, 64) */
+                           bits 8-23: KiB per tile and round for order 4 (0 = default: 64 for copy groups, 4 for span groups) */
 } mmr_plan_options;
 
 typedef struct {
