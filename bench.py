@@ -45,10 +45,11 @@ def kernel_sources_digest():
     sources says nothing about this build."""
     h = hashlib.sha256()
     base = os.path.join(ROOT, "multimesh-jax_amd", "csrc")
-    for name in sorted(os.listdir(base)):
-        if name.endswith((".hip", ".h", ".cc")):
-            with open(os.path.join(base, name), "rb") as f:
-                h.update(name.encode() + b"\0" + f.read())
+    # the kernels, the per-workgroup code and the planner (what decides which bytes a launch touches); not the host
+    # code around them
+    for name in ("chunk_ops.h", "geometry.cc", "group_ops.h", "kernels.h", "kernels.hip", "planner.cc", "planner.h"):
+        with open(os.path.join(base, name), "rb") as f:
+            h.update(name.encode() + b"\0" + f.read())
     return h.hexdigest()[:16]
 
 

@@ -278,6 +278,15 @@ int check_spans(const mmr_plan& plan) {
     if (g.span == 0 || g.span > mmr::kSpanMaxBytes || g.head == 0 || g.head > g.span || g.W == 0 ||
         g.W > mmr::kSpanMaxRowBytes)
       return fail(MMR_INTERNAL, "span group with span %u, head %u, row %u", g.span, g.head, g.W);
+  // a group that uses the segment table: one lane per (row, piece) pair that can touch a span
+  for (const mmr::SpanGroup& g : plan.span_groups) {
+    if (!g.table_mode) continue;
+    for (uint32_t t = 0; t < g.il.members; ++t) {
+      const mmr::SpanMember& m = plan.span_members[g.first_member + t];
+      if (m.k == 0 || m.k > mmr::kSpanTablePieces || (static_cast<uint64_t>(g.span) / g.W + 2) * m.k > mmr::kSpanLanes)
+        return fail(MMR_INTERNAL, "span group with %u pieces per row of %u bytes cannot use a segment table", m.k, g.W);
+    }
+  }
   return MMR_OK;
 }
 
