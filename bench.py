@@ -177,10 +177,10 @@ def measure(ctx, mm, workloads, args, config):
     ctx.StartTimer()
     for i in range(args.steps):
         step(i)
-    kernel_ms = ctx.StopTimer()
+    syncs_in_region = ctx.stats["host_blocking_syncs"] - syncs_before  # waits the K reshards themselves caused
+    kernel_ms = ctx.StopTimer()  # blocks until the device gets there (a counted wait, asked for here)
     ctx.Sync()
     wall_s = time.perf_counter() - t0
-    syncs_in_region = ctx.stats["host_blocking_syncs"] - syncs_before
     # the same bracket five more times over 50 back-to-back launches each: the median of the five means
     brackets = []
     for _ in range(5):
@@ -286,9 +286,44 @@ def record_traffic(args):
     print(json.dumps(prof))
 
 
+def through_context(result, others):
+    """The same reshards behind the reference-shaped interface: tests/cpp/context_bench builds configurations 2 and
+    4 as a ReshardSchedule and runs ReshardSchedule::Execute over HipExecuteContext with 12 local devices (one Reshard
+    call per array and local device, fresh root stores and the OpenWindow / StartTimer / ... / CloseWindow bracket
+    every execution).  Each runs as a child process of its own, started after this process has closed its context."""
+    import subprocess
+    exe = os.path.join(ROOT, "tests", "cpp", "context_bench")
+    if not os.path.exists(exe):
+        return {"error": "tests/cpp/context_bench is not built (tests/cpp/build.sh)"}
+    direct = {2: result if result["config"]["workload"].startswith("configuration 2") else others.get("config2"),
+              4: others.get("config4")}
+    out = {}
+    for config, executions in ((2, 100), (4, 30)):
+        try:
+            p = subprocess.run([exe, str(config), str(executions)], capture_output=True, text=True, timeout=240)
+        except subprocess.TimeoutExpired:
+            out["config%d" % config] = {"error": "timed out"}
+            continue
+        if p.returncode != 0:
+            out["config%d" % config] = {"error": (p.stdout + p.stderr)[-400:], "returncode": p.returncode}
+            continue
+        r = json.loads(p.stdout.strip().splitlines()[-1])
+        d = direct.get(config)
+        if d is not None:
+            direct_ms = d["ms_per_step"]
+            direct_kernel_ms = d["roofline"]["kernel_ms"] if "roofline" in d else d["kernel_ms"]
+            r["direct_c_abi_ms_per_step"] = direct_ms
+            r["direct_c_abi_kernel_ms"] = direct_kernel_ms
+            r["wall_over_direct"] = round(r["wall_ms_per_execution"] / direct_ms, 4)
+            r["host_ms_over_kernel_ms"] = round(r["host_ms_per_execute_median"] / direct_kernel_ms, 4)
+        out["config%d" % config] = r
+    return out
+
+
 def summary(r):
     return {"GB/s": round(r["achieved"], 1), "frac_hbm_peak": round(r["achieved"] / HBM_PEAK_GBS, 4),
-            "kernel_ms": round(r["kernel_ms"], 5), "median_ms": round(r["median_ms"], 5),
+            "kernel_ms": round(r["kernel_ms"], 5), "ms_per_step": round(r["ms_per_step"], 5),
+            "wall_GB/s": round(r["value"], 1), "median_ms": round(r["median_ms"], 5),
             "p10_ms": round(r["p10_ms"], 5), "p90_ms": round(r["p90_ms"], 5), "launches_timed": r["laps"],
             "bracket_median_ms": round(r["bracket_median_ms"], 5),
             "median_GB/s": round(r["median_gbs"], 1), "algorithmic_bytes": r["alg_bytes"],
@@ -307,6 +342,8 @@ def main():
     ap.add_argument("--only", action="store_true", help="measure --config alone (no all_configs)")
     ap.add_argument("--all", action="store_true", help="accepted for compatibility: all_configs is the default")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-through-context", action="store_true",
+                    help="skip the child runs that time configurations 2 and 4 through ReshardSchedule::Execute")
     ap.add_argument("--no-tune", dest="tune", action="store_false",
                     help="keep the planner's default launch order instead of timing a few on the first buffer set")
     ap.add_argument("--unbatched", action="store_true",
@@ -426,6 +463,8 @@ def main():
             ctx.ClearStoreCache()
         result["all_configs"] = others
     ctx.close()
+    if not args.only and not args.workload_json and args.scale == 1 and not args.name and not args.no_through_context:
+        result["through_context"] = through_context(result, others if "all_configs" in result else {})
     print(json.dumps(result))
 
 

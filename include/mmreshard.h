@@ -270,6 +270,9 @@ int mmr_context_set_plan_options(mmr_context* ctx, const mmr_plan_options* optio
  * descriptors; mm_mock_mm_xla.cc:259-262, compared between runs at mm_pjrt_executable_test.cc:760-766) and, on every
  * reshard, "every operand holds a tile on each of its devices" (mm_mock_mm_xla.cc:347-369).  Off by default. */
 #define MMR_CHECK_INVARIANTS 1u
+/* Every named timer that completes prints "<name> finished in <seconds>s" to stderr, the line the reference logs at
+ * info level (zuku_execute_context_impl.cc:478-482). */
+#define MMR_LOG_TIMERS 2u
 int mmr_context_set_flags(mmr_context* ctx, uint32_t flags);
 
 #define MMR_STORE_FROM_CACHE 1u    /* CreateStoreConfig::allocate_from_cache */
@@ -371,13 +374,17 @@ int mmr_reshard_bind(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const*
 int mmr_reshard_validate(mmr_context* ctx, mmr_store* src, mmr_store* dst);
 
 /* No counterpart in the reference.  For callers that cannot allocate device memory where they reshard: code that
- * runs under HIP graph capture, tight serving loops, harnesses that forbid allocation.  Does what mmr_reshard_batch does,
+ * runs in tight serving loops or under harnesses that forbid allocation.  Does what mmr_reshard_batch does,
  * with the same kernels, but the chunk tables and the table of shard pointers of the launch live in a static device
  * array of MMR_STATIC_SCRATCH_BYTES per GPU instead of allocated memory: the call plans on the host, copies the tables
  * into that array on the context's stream (through a pinned staging buffer the context has held since its creation)
- * and launches; it calls no hipMalloc / hipFree.  A plan whose tables exceed the array is refused with MMR_INVALID_ARGUMENT (use mmr_reshard_batch).  Every
- * call on a GPU shares that GPU's array: calls are safe one after the other on one stream, calls that overlap on one GPU
- * (two contexts, two streams) race.  No table order tuning. */
+ * and launches; it calls no hipMalloc / hipFree.  A plan whose tables exceed the array is refused with MMR_INVALID_ARGUMENT (use mmr_reshard_batch).
+ * It copies from host memory, so like every such entry point it is refused (MMR_INVALID_ARGUMENT, capture left
+ * valid) while the context's stream is capturing a graph: a capturable reshard is mmr_reshard_bind + mmr_reshard.
+ * Every call on a GPU shares that GPU's array.  Calls of one context follow each other on its stream; a call of
+ * another context of this process on the same GPU makes its stream wait, on the device, for the kernels of the
+ * previous user.  Streams of other processes and callers that bypass this entry point are not ordered: such calls
+ * race.  No table order tuning. */
 #define MMR_STATIC_SCRATCH_BYTES (1u << 20)
 int mmr_reshard_batch_static(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int32_t n);
 
@@ -403,18 +410,57 @@ int mmr_context_prepare(mmr_context* ctx, const mmr_sharded_shape* srcs, const m
 int mmr_context_wait_event(mmr_context* ctx, void* hip_event);
 int mmr_context_record_event(mmr_context* ctx, void* hip_event);
 
-/* RunAfterAllTasks, zuku_execute_context.h:53-54, zuku_execute_context_impl.cc:347-354: fn(arg) runs on a runtime
- * thread once everything queued on the context's stream so far is done; the call itself does not wait.  fn must not
- * call into this library. */
+/* RunAfterAllTasks, zuku_execute_context.h:53-54, zuku_execute_context_impl.cc:347-354: fn(arg) runs once everything
+ * queued on the context's stream so far is done; the call itself does not wait.  fn runs on a thread the context
+ * owns (never on a thread of the HIP runtime), callbacks run one at a time in the order they were given, and fn may
+ * call any entry point of this library except mmr_context_destroy - the reference's callback completes a future whose
+ * continuations drop buffers (mm_pjrt_executable.cc:373-375).  mmr_context_destroy runs the callbacks still waiting
+ * before it returns. */
 int mmr_context_run_after(mmr_context* ctx, void (*fn)(void*), void* arg);
 
-/* Blocks until everything queued on the context's stream is done. */
+/* Blocks until everything queued on the context's stream is done and the callbacks of mmr_context_run_after given
+ * before this call have returned (called from such a callback, it only waits for the stream). */
 int mmr_sync(mmr_context* ctx);
 
-/* HIP-event timing on the context's stream (StartTimer/StopTimer,
- * zuku_execute_context_impl.cc:462-486, measure wall clock; here device time). */
+/* StartTimer / StopTimer, zuku_execute_context.h:56-59, zuku_execute_context_impl.cc:462-486: named timers, any
+ * number pending at once, and neither call waits for the device.  The reference defers a steady_clock reading
+ * behind the last execute event on both sides and logs the difference from a deferred task; here both sides are
+ * HIP events on the context's stream, so the interval is the device time between the two points.
+ * mmr_timer_begin: a timer of that name that is already running is left as it is (pending_timers_.emplace, :466).
+ * mmr_timer_end: MMR_NOT_FOUND if no such timer is running (the reference logs a warning and goes on, :471-474).
+ * An interval is read once the device has passed its end, by whichever of these calls (or mmr_window_open) comes
+ * next; mmr_timer_poll never waits: *last_milliseconds is the most recent interval of `name` that has been read
+ * (0 if none), *completed how many have been.  mmr_timer_wait is the blocking variant: it first waits until every
+ * ended interval of `name` has been read (counted in host_blocking_syncs when it has to wait). */
+int mmr_timer_begin(mmr_context* ctx, const char* name);
+int mmr_timer_end(mmr_context* ctx, const char* name);
+int mmr_timer_poll(mmr_context* ctx, const char* name, float* last_milliseconds, int64_t* completed);
+int mmr_timer_wait(mmr_context* ctx, const char* name, float* last_milliseconds, int64_t* completed);
+
+/* MarkProfile, zuku_execute_context.h:55, zuku_execute_context_impl.cc:458-460: a named mark in the profile.  Goes
+ * out as a roctx marker (rocprofv3 --marker-trace shows it); the library also wraps plan building, table binding and
+ * every launch of a reshard in roctx ranges ("mmreshard: build plan" / "bind tables" / "launch"), the counterpart of
+ * the named region around every task of the reference (:292-308).  The roctx library is looked up at run time
+ * (librocprofiler-sdk-roctx, then libroctx64); where neither is installed, or with MMR_ROCTX=0 in the environment,
+ * the calls do nothing.  mmr_profile_available: 1 if marks reach a roctx library. */
+int mmr_profile_mark(mmr_context* ctx, const char* name);
+int mmr_profile_range_push(mmr_context* ctx, const char* name);
+int mmr_profile_range_pop(mmr_context* ctx);
+int mmr_profile_available(void);
+
+/* OpenWindow / CloseWindow, zuku_execute_context.h:50-51, zuku_execute_context_impl.cc:128-143: one window per
+ * execution of an executable (mm_pjrt_executable.cc:362, 705).  mmr_window_close marks the end of everything queued
+ * so far; mmr_window_open returns at once while fewer than the limit (8, kMaxOpenWindows, :46) windows are still
+ * running on the device and otherwise waits for the oldest one (counted in window_waits and host_blocking_syncs), so
+ * a caller that never reads a result cannot run ahead of the device without bound.  (In the reference tree the line
+ * that queues the marker, :140, is commented out, so its limit never triggers; the limit it declares is kept here.) */
+int mmr_window_open(mmr_context* ctx);
+int mmr_window_close(mmr_context* ctx);
+int mmr_context_set_max_open_windows(mmr_context* ctx, int32_t n);
+
+/* Unnamed HIP-event stopwatch on the context's stream for benchmarks: one interval at a time. */
 int mmr_timer_start(mmr_context* ctx);
-int mmr_timer_stop(mmr_context* ctx, float* milliseconds); /* blocks */
+int mmr_timer_stop_wait(mmr_context* ctx, float* milliseconds); /* blocks until the device reaches this point */
 /* Per-launch timing of back-to-back work: mmr_timer_lap records a mark on the stream (between two launches, say);
  * mmr_timer_laps blocks until the last mark is reached, writes the device time between consecutive marks
  * (marks - 1 values, at most `capacity`; *count = how many) and forgets the marks. */
@@ -434,7 +480,8 @@ typedef struct {
   int64_t cache_hits;      /* store buffers served from the per-shape cache */
   int64_t host_bytes_allocated; /* pinned host bytes of offloaded stores and of the host cache */
   int64_t host_bytes_high_watermark;
-  int64_t host_blocking_syncs;  /* times an entry point made the calling thread wait for the device */
+  int64_t host_blocking_syncs;  /* times an entry point made the calling thread wait for the device: every
+                                   stream / event synchronisation and every hipFree the library issues */
   int64_t inline_launches;      /* launches whose table travelled in the kernel's argument block */
   int64_t device_allocations;   /* hipMalloc calls */
   int64_t host_cache_hits;      /* offloads served from the pinned host cache */
@@ -443,6 +490,11 @@ typedef struct {
   int64_t bindings_cached;      /* bound device tables held now */
   int64_t invariant_checks;     /* checks made in MMR_CHECK_INVARIANTS mode */
   int64_t operation_hash;       /* rolling hash of the operation stream in that mode */
+  int64_t block_pool_hits;      /* table blocks (plans, bindings) served from the pool of recycled blocks */
+  int64_t timers_resolved;      /* named timer intervals read so far */
+  int64_t windows_opened;
+  int64_t window_waits;         /* mmr_window_open calls that had to wait for an older window */
+  int64_t profile_marks;
 } mmr_context_stats;
 int mmr_context_get_stats(mmr_context* ctx, mmr_context_stats* out);
 /* Stats of the cached plan of a store pair (builds it if needed). */

@@ -101,8 +101,11 @@ class HipExecuteContextAdapter : public ZukuExecuteContext {
   }
 
   void Destroy(StoreHandle& store) override {
-    if (store.impl != nullptr) ctx_->Destroy(store.impl->inner);
-    store.impl = nullptr;  // zuku_execute_context_impl.cc:356-361
+    // Drops the caller's reference only (zuku_execute_context_impl.cc:356-361).  The impl is shared by every copy of
+    // the handle - ~MultiMeshPjRtBuffer calls Destroy while a StoreExternalReference (mm_pjrt_buffer.cc:27-36) may
+    // still hold a copy to keep the tile of a zero-copy view alive - so the library's handle inside it is released
+    // only when the last copy goes.
+    store.impl = nullptr;
   }
 
   void ClearStoreCache(int64_t local_device_id) override {
@@ -126,14 +129,20 @@ class HipExecuteContextAdapter : public ZukuExecuteContext {
   }
 
   // ---- windows, ordering, profiling ---------------------------------------------------------------------------
-  void OpenWindow() override { ctx_->OpenWindow(); }
+  void OpenWindow() override {
+    Guard([&] { ctx_->OpenWindow(); });  // waits only while 8 earlier windows are still running on the device
+  }
   void CloseWindow() override {
     Guard([&] { ctx_->CloseWindow(); });  // the reshards queued for the window leave here at the latest
   }
   void RunAfterAllTasks(int64_t local_device_id, std::function<void()> on_done) override {
+    // on_done runs on a thread the library owns, never on a HIP runtime thread: it may complete a PjRtFuture whose
+    // continuations drop buffers and so call back into this context (mm_pjrt_executable.cc:373-375)
     Guard([&] { ctx_->RunAfterAllTasks(local_device_id, std::move(on_done)); });
   }
-  void MarkProfile(const std::string& name) override { ctx_->MarkProfile(name); }
+  void MarkProfile(const std::string& name) override {
+    Guard([&] { ctx_->MarkProfile(name); });
+  }
   void StartTimer(const std::string& name) override {
     Guard([&] { ctx_->StartTimer(name); });
   }

@@ -99,7 +99,7 @@ class ContextStats(C.Structure):
         "reshard_calls", "bytes_allocated", "bytes_high_watermark", "stores_live", "cache_hits",
         "host_bytes_allocated", "host_bytes_high_watermark", "host_blocking_syncs", "inline_launches",
         "device_allocations", "host_cache_hits", "pool_hits", "plans_cached", "bindings_cached", "invariant_checks",
-        "operation_hash")]
+        "operation_hash", "block_pool_hits", "timers_resolved", "windows_opened", "window_waits", "profile_marks")]
 
     def as_dict(self):
         return {n: getattr(self, n) for n, _ in self._fields_}
@@ -171,7 +171,18 @@ PROTOTYPES = {
     "mmr_context_run_after": (C.c_int, [VP, C.CFUNCTYPE(None, VP), VP]),
     "mmr_sync": (C.c_int, [VP]),
     "mmr_timer_start": (C.c_int, [VP]),
-    "mmr_timer_stop": (C.c_int, [VP, P(C.c_float)]),
+    "mmr_timer_stop_wait": (C.c_int, [VP, P(C.c_float)]),
+    "mmr_timer_begin": (C.c_int, [VP, C.c_char_p]),
+    "mmr_timer_end": (C.c_int, [VP, C.c_char_p]),
+    "mmr_timer_poll": (C.c_int, [VP, C.c_char_p, P(C.c_float), P(I64)]),
+    "mmr_timer_wait": (C.c_int, [VP, C.c_char_p, P(C.c_float), P(I64)]),
+    "mmr_profile_mark": (C.c_int, [VP, C.c_char_p]),
+    "mmr_profile_range_push": (C.c_int, [VP, C.c_char_p]),
+    "mmr_profile_range_pop": (C.c_int, [VP]),
+    "mmr_profile_available": (C.c_int, []),
+    "mmr_window_open": (C.c_int, [VP]),
+    "mmr_window_close": (C.c_int, [VP]),
+    "mmr_context_set_max_open_windows": (C.c_int, [VP, I32]),
     "mmr_timer_lap": (C.c_int, [VP]),
     "mmr_timer_laps": (C.c_int, [VP, P(C.c_float), I32, P(I32)]),
     "mmr_context_get_stats": (C.c_int, [VP, P(ContextStats)]),

@@ -507,13 +507,48 @@ class ReshardContext:
         opt = B.PlanOptions(chunk_bytes, order, xcd_mode, flags)
         B.check(self._lib.mmr_context_set_plan_options(self._h, C.byref(opt)))
 
-    def StartTimer(self) -> None:
-        B.check(self._lib.mmr_timer_start(self._h))
+    def StartTimer(self, name: Optional[str] = None) -> None:
+        """StartTimer(name) of the reference (zuku_execute_context_impl.cc:462-467): named, any number pending, does
+        not wait.  Without a name: the unnamed benchmark stopwatch (one interval at a time)."""
+        if name is None:
+            B.check(self._lib.mmr_timer_start(self._h))
+        else:
+            B.check(self._lib.mmr_timer_begin(self._h, name.encode()))
 
-    def StopTimer(self) -> float:
-        ms = C.c_float()
-        B.check(self._lib.mmr_timer_stop(self._h, C.byref(ms)))
-        return ms.value
+    def StopTimer(self, name: Optional[str] = None) -> Optional[float]:
+        """StopTimer(name) (:469-486): does not wait; an unknown name is a warning as in the reference.  Without a
+        name: stops the benchmark stopwatch, BLOCKS until the device gets there and returns milliseconds."""
+        if name is None:
+            ms = C.c_float()
+            B.check(self._lib.mmr_timer_stop_wait(self._h, C.byref(ms)))
+            return ms.value
+        rc = self._lib.mmr_timer_end(self._h, name.encode())
+        if rc == 5:  # MMR_NOT_FOUND
+            import warnings
+            warnings.warn(self._lib.mmr_last_error().decode("utf-8", "replace"))
+            return None
+        B.check(rc)
+        return None
+
+    def TimerResult(self, name: str, wait: bool = False):
+        """(milliseconds of the most recent completed interval of `name`, intervals completed).  Never waits unless
+        `wait` is set."""
+        ms, n = C.c_float(), C.c_int64()
+        fn = self._lib.mmr_timer_wait if wait else self._lib.mmr_timer_poll
+        B.check(fn(self._h, name.encode(), C.byref(ms), C.byref(n)))
+        return ms.value, n.value
+
+    def MarkProfile(self, name: str) -> None:
+        B.check(self._lib.mmr_profile_mark(self._h, name.encode()))
+
+    def OpenWindow(self) -> None:
+        B.check(self._lib.mmr_window_open(self._h))
+
+    def CloseWindow(self) -> None:
+        B.check(self._lib.mmr_window_close(self._h))
+
+    def set_max_open_windows(self, n: int) -> None:
+        B.check(self._lib.mmr_context_set_max_open_windows(self._h, n))
 
     def Lap(self) -> None:
         """A timing mark on the stream (see Laps)."""

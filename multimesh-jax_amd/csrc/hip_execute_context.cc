@@ -3,6 +3,7 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <cstdio>
 #include <stdexcept>
 
 namespace mmr {
@@ -98,42 +99,66 @@ void require_live(const StoreHandle& h, const char* where) {
 std::shared_ptr<HipExecuteContext> HipExecuteContext::Create(std::set<int> local_devices, int hip_device) {
   std::shared_ptr<HipExecuteContext> c(new HipExecuteContext());
   if (local_devices.empty()) raise("HipExecuteContext::Create: no local devices");
+  if (*local_devices.begin() < 0) raise("HipExecuteContext::Create: negative local device id");
   c->local_devices_ = std::move(local_devices);
+  c->position_of_.assign(static_cast<size_t>(*c->local_devices_.rbegin()) + 1, -1);
+  int32_t position = 0;
+  for (int d : c->local_devices_) c->position_of_[static_cast<size_t>(d)] = position++;
+  for (OpStream& s : c->streams_) s.next_seq.assign(c->local_devices_.size(), 0);
   check(mmr_context_create(hip_device, nullptr, &c->ctx_), "HipExecuteContext::Create");
   return c;
 }
 
 HipExecuteContext::~HipExecuteContext() {
-  pending_.clear();    // work nobody waited for
-  in_flight_.clear();  // drops the stores still attached to half-arrived ops
+  pending_.clear();  // work nobody waited for
+  for (OpStream& s : streams_) s.ops.clear();  // drops the stores still attached to half-arrived ops
   // Handles may outlive the context (Python shutdown order in the reference,
   // zuku_execute_context_impl.cc:64-71); their stores die with the context.
   alive_->store(false);
-  if (ctx_) mmr_context_destroy(ctx_);
+  if (ctx_) mmr_context_destroy(ctx_);  // runs the callbacks of RunAfterAllTasks that are still waiting
 }
 
-HipExecuteContext::ReplicatedOp& HipExecuteContext::Arrive(const char* kind, int64_t local_device_id, bool* first) {
-  if (!local_devices_.count(static_cast<int>(local_device_id)))
-    raise(std::string(kind) + ": device " + std::to_string(local_device_id) + " is not a local device");
-  const int64_t seq = next_seq_[kind][local_device_id]++;
-  auto& ops = in_flight_[kind];
-  auto it = ops.find(seq);
-  *first = it == ops.end();
-  ReplicatedOp& op = ops[seq];
+namespace {
+const char* const kOpNames[] = {"CreateStore", "Reshard", "OffloadDtoH", "OffloadHtoD"};
+}
+
+HipExecuteContext::ReplicatedOp& HipExecuteContext::Arrive(OpKind kind, int64_t local_device_id, bool* first, int64_t* seq) {
+  if (local_device_id < 0 || local_device_id >= static_cast<int64_t>(position_of_.size()) ||
+      position_of_[static_cast<size_t>(local_device_id)] < 0)
+    raise(std::string(kOpNames[kind]) + ": device " + std::to_string(local_device_id) + " is not a local device");
+  OpStream& s = streams_[kind];
+  *seq = s.next_seq[static_cast<size_t>(position_of_[static_cast<size_t>(local_device_id)])]++;
+  const int64_t at = *seq - s.first_seq;  // >= 0: an op leaves the front only after every device has issued it
+  *first = at == static_cast<int64_t>(s.ops.size());
+  if (at > static_cast<int64_t>(s.ops.size()))
+    raise(std::string(kOpNames[kind]) + ": call order between local devices is inconsistent");
+  if (*first) s.ops.emplace_back();
+  ReplicatedOp& op = s.ops[static_cast<size_t>(at)];
   op.arrivals += 1;
   return op;
 }
 
-void HipExecuteContext::Leave(const char* kind, int64_t seq, const ReplicatedOp& op) {
-  if (op.arrivals == static_cast<int>(local_devices_.size())) in_flight_[kind].erase(seq);
+void HipExecuteContext::Leave(OpKind kind) {
+  OpStream& s = streams_[kind];
+  const int n = static_cast<int>(local_devices_.size());
+  while (!s.ops.empty() && s.ops.front().arrivals == n) {
+    s.ops.pop_front();
+    s.first_seq += 1;
+  }
+}
+
+void HipExecuteContext::Retract(OpKind kind, int64_t local_device_id) {
+  OpStream& s = streams_[kind];
+  s.ops.pop_back();
+  s.next_seq[static_cast<size_t>(position_of_[static_cast<size_t>(local_device_id)])]--;
 }
 
 StoreHandle HipExecuteContext::CreateStore(int64_t local_device_id, int64_t global_device_id, ShardedShape shape,
                                            CreateStoreConfig config) {
   std::lock_guard<std::mutex> lock(mu_);
   bool first = false;
-  const int64_t seq = next_seq_["CreateStore"][local_device_id];
-  ReplicatedOp& op = Arrive("CreateStore", local_device_id, &first);
+  int64_t seq = 0;
+  ReplicatedOp& op = Arrive(kCreateStore, local_device_id, &first, &seq);
   if (first) {
     auto shared = std::make_shared<SharedStore>();
     shared->ctx = ctx_;
@@ -145,8 +170,7 @@ StoreHandle HipExecuteContext::CreateStore(int64_t local_device_id, int64_t glob
                            (config.uninitialized ? MMR_STORE_UNINITIALIZED : 0u);
     int rc = mmr_store_create_ex(ctx_, &pod, name, flags, config.min_cache_size.value_or(1), &shared->store);
     if (rc != MMR_OK) {
-      in_flight_["CreateStore"].erase(seq);
-      next_seq_["CreateStore"][local_device_id]--;
+      Retract(kCreateStore, local_device_id);
       check(rc, "CreateStore");
     }
     op.store = shared;
@@ -161,7 +185,7 @@ StoreHandle HipExecuteContext::CreateStore(int64_t local_device_id, int64_t glob
   handle.impl->local_device_id = local_device_id;
   handle.impl->global_device_id = global_device_id;
   handle.unique_id = mmr_store_id(op.store->store);
-  Leave("CreateStore", seq, op);
+  Leave(kCreateStore);
   return handle;
 }
 
@@ -191,8 +215,8 @@ void HipExecuteContext::Reshard(int64_t local_device_id, int64_t global_device_i
   require_live(dst, "Reshard");
   std::lock_guard<std::mutex> lock(mu_);
   bool first = false;
-  const int64_t seq = next_seq_["Reshard"][local_device_id];
-  ReplicatedOp& op = Arrive("Reshard", local_device_id, &first);
+  int64_t seq = 0;
+  ReplicatedOp& op = Arrive(kReshard, local_device_id, &first, &seq);
   const int64_t s = src.unique_id, d = dst.unique_id;
   if (first) {
     op.a = s;
@@ -202,44 +226,49 @@ void HipExecuteContext::Reshard(int64_t local_device_id, int64_t global_device_i
     std::shared_ptr<SharedStore> sa = src.impl->array, da = dst.impl->array;
     int rc = mmr_reshard_validate(ctx_, sa->store, da->store);
     if (rc == MMR_OK && defer_reshards_) {
-      bool depends = false;
-      for (const auto& q : pending_)
-        depends |= q.second == sa || q.second == da || q.first == da;  // reads or overwrites a queued result / input
+      // reads or overwrites a queued result, or overwrites a queued input
+      const bool depends = pending_dsts_.count(sa.get()) || pending_dsts_.count(da.get()) || pending_srcs_.count(da.get());
       try {
         if (depends) FlushLocked();
       } catch (...) {
-        in_flight_["Reshard"].erase(seq);
-        next_seq_["Reshard"][local_device_id]--;
+        Retract(kReshard, local_device_id);
         throw;
       }
+      pending_srcs_.insert(sa.get());
+      pending_dsts_.insert(da.get());
       pending_.emplace_back(std::move(sa), std::move(da));
     } else if (rc == MMR_OK) {
       rc = mmr_reshard(ctx_, sa->store, da->store);
     }
     if (rc != MMR_OK) {
-      in_flight_["Reshard"].erase(seq);
-      next_seq_["Reshard"][local_device_id]--;
+      Retract(kReshard, local_device_id);
       check(rc, "Reshard");
     }
   } else if (op.a != s || op.b != d) {
     raise("Reshard: device " + std::to_string(local_device_id) + " issues reshard #" + std::to_string(seq) +
           " on different stores than the device that started it (control replication broken)");
   }
-  Leave("Reshard", seq, op);
+  Leave(kReshard);
 }
 
 void HipExecuteContext::FlushLocked() {
   if (pending_.empty()) return;
-  std::vector<mmr_store*> srcs, dsts;
+  flush_srcs_.clear();
+  flush_dsts_.clear();
   for (const auto& q : pending_) {
-    srcs.push_back(q.first->store);
-    dsts.push_back(q.second->store);
+    flush_srcs_.push_back(q.first->store);
+    flush_dsts_.push_back(q.second->store);
   }
   auto keep = std::move(pending_);  // the stores stay alive until the launches are issued; a failure is not retried
   pending_.clear();
-  check(srcs.size() == 1 ? mmr_reshard(ctx_, srcs[0], dsts[0])
-                         : mmr_reshard_batch(ctx_, srcs.data(), dsts.data(), static_cast<int32_t>(srcs.size())),
-        "Reshard");
+  pending_srcs_.clear();
+  pending_dsts_.clear();
+  (void)mmr_profile_range_push(ctx_, "HipExecuteContext: reshards of a window");  // the named region of a task
+  const int rc = flush_srcs_.size() == 1
+                     ? mmr_reshard(ctx_, flush_srcs_[0], flush_dsts_[0])
+                     : mmr_reshard_batch(ctx_, flush_srcs_.data(), flush_dsts_.data(), static_cast<int32_t>(flush_srcs_.size()));
+  (void)mmr_profile_range_pop(ctx_);
+  check(rc, "Reshard");
 }
 
 void HipExecuteContext::Flush() {
@@ -323,8 +352,8 @@ void HipExecuteContext::OffloadDtoH(int64_t local_device_id, const std::vector<S
   (void)task_name;
   std::lock_guard<std::mutex> lock(mu_);
   bool first = false;
-  const int64_t seq = next_seq_["OffloadDtoH"][local_device_id];
-  ReplicatedOp& op = Arrive("OffloadDtoH", local_device_id, &first);
+  int64_t seq = 0;
+  (void)Arrive(kOffloadDtoH, local_device_id, &first, &seq);
   if (first) {
     FlushLocked();
     for (const StoreHandle& h : to_offload) {
@@ -332,7 +361,7 @@ void HipExecuteContext::OffloadDtoH(int64_t local_device_id, const std::vector<S
       check(mmr_store_offload(ctx_, h.impl->array->store), "OffloadDtoH");
     }
   }
-  Leave("OffloadDtoH", seq, op);
+  Leave(kOffloadDtoH);
 }
 
 void HipExecuteContext::OffloadHtoD(int64_t local_device_id, const std::vector<StoreHandle>& to_offload,
@@ -340,8 +369,8 @@ void HipExecuteContext::OffloadHtoD(int64_t local_device_id, const std::vector<S
   (void)task_name;
   std::lock_guard<std::mutex> lock(mu_);
   bool first = false;
-  const int64_t seq = next_seq_["OffloadHtoD"][local_device_id];
-  ReplicatedOp& op = Arrive("OffloadHtoD", local_device_id, &first);
+  int64_t seq = 0;
+  (void)Arrive(kOffloadHtoD, local_device_id, &first, &seq);
   if (first) {
     FlushLocked();
     for (const StoreHandle& h : to_offload) {
@@ -349,10 +378,17 @@ void HipExecuteContext::OffloadHtoD(int64_t local_device_id, const std::vector<S
       check(mmr_store_reload(ctx_, h.impl->array->store), "OffloadHtoD");
     }
   }
-  Leave("OffloadHtoD", seq, op);
+  Leave(kOffloadHtoD);
 }
 
-void HipExecuteContext::CloseWindow() { Flush(); }
+void HipExecuteContext::OpenWindow() { check(mmr_window_open(ctx_), "OpenWindow"); }
+
+void HipExecuteContext::CloseWindow() {
+  Flush();
+  check(mmr_window_close(ctx_), "CloseWindow");
+}
+
+void HipExecuteContext::SetMaxOpenWindows(int n) { check(mmr_context_set_max_open_windows(ctx_, n), "SetMaxOpenWindows"); }
 
 void HipExecuteContext::RunAfterAllTasks(int64_t local_device_id, std::function<void()> on_done) {
   (void)local_device_id;
@@ -374,22 +410,36 @@ void HipExecuteContext::RunAfterAllTasks(int64_t local_device_id, std::function<
   }
 }
 
-void HipExecuteContext::MarkProfile(const std::string& name) { (void)name; }
+void HipExecuteContext::MarkProfile(const std::string& name) { check(mmr_profile_mark(ctx_, name.c_str()), "MarkProfile"); }
 
 void HipExecuteContext::StartTimer(const std::string& name) {
-  (void)name;
-  Flush();
-  check(mmr_timer_start(ctx_), "StartTimer");
+  Flush();  // the timer starts behind the work issued so far
+  check(mmr_timer_begin(ctx_, name.c_str()), "StartTimer");
 }
 
 void HipExecuteContext::StopTimer(const std::string& name) {
-  float ms = 0;
   Flush();
-  check(mmr_timer_stop(ctx_, &ms), "StopTimer");
-  timers_ms_[name] = ms;
+  const int rc = mmr_timer_end(ctx_, name.c_str());
+  if (rc == MMR_NOT_FOUND) {  // zuku_execute_context_impl.cc:471-474: a warning, not an error
+    std::fprintf(stderr, "warning: %s\n", mmr_last_error());
+    return;
+  }
+  check(rc, "StopTimer");
 }
 
-double HipExecuteContext::LastTimerMilliseconds(const std::string& name) { return timers_ms_[name]; }
+double HipExecuteContext::LastTimerMilliseconds(const std::string& name, int64_t* completed) {
+  float ms = 0;
+  int64_t n = 0;
+  check(mmr_timer_poll(ctx_, name.c_str(), &ms, &n), "LastTimerMilliseconds");
+  if (completed) *completed = n;
+  return ms;
+}
+
+double HipExecuteContext::WaitTimerMilliseconds(const std::string& name) {
+  float ms = 0;
+  check(mmr_timer_wait(ctx_, name.c_str(), &ms, nullptr), "WaitTimerMilliseconds");
+  return ms;
+}
 
 mmr_context_stats HipExecuteContext::Stats() {
   Flush();
@@ -421,13 +471,23 @@ void ReshardSchedule::AddReshardTask(const Store& input, const Store& output) {
 }
 
 std::vector<std::vector<StoreHandle>> ReshardSchedule::Execute(
-    HipExecuteContext& ctx, const std::vector<std::vector<StoreHandle>>& parameter_stores) {
+    HipExecuteContext& ctx, const std::vector<std::vector<StoreHandle>>& parameter_stores,
+    std::vector<std::function<void()>>* on_done) {
   const std::set<int> local = ctx.GetLocalDevices();
   const std::vector<int> devices(local.begin(), local.end());
   const size_t n = devices.size();
   if (parameter_stores.size() != n) raise("Execute: one list of parameter stores per local device is required");
   for (const auto& p : parameter_stores)
     if (static_cast<int64_t>(p.size()) != num_params_) raise("Execute: wrong number of parameter stores");
+  if (on_done && !on_done->empty() && on_done->size() != n) raise("Execute: one callback per local device is required");
+  if (start_mark_.empty()) {
+    start_mark_ = "start " + name_;
+    finish_mark_ = "finish " + name_;
+  }
+  // mm_pjrt_executable.cc:362-364
+  ctx.OpenWindow();
+  ctx.StartTimer(name_);
+  ctx.MarkProfile(start_mark_);
   std::vector<std::vector<StoreHandle>> root_stores(n, std::vector<StoreHandle>(static_cast<size_t>(num_roots_)));
   for (const MpmdOperation& op : schedule_) {  // add_root_store: once per root, for every local device
     const Store& out = op.op.output;
@@ -453,6 +513,12 @@ std::vector<std::vector<StoreHandle>> ReshardSchedule::Execute(
   for (const MpmdOperation& op : schedule_)
     for (size_t i = 0; i < n; ++i)
       ctx.Reshard(devices[i], devices[i], handle_of(i, op.op.input), handle_of(i, op.op.output));
+  if (on_done && !on_done->empty())  // :660-667
+    for (size_t i = 0; i < n; ++i) ctx.RunAfterAllTasks(devices[i], std::move((*on_done)[i]));
+  // :704-706
+  ctx.StopTimer(name_);
+  ctx.CloseWindow();
+  ctx.MarkProfile(finish_mark_);
   return root_stores;
 }
 

@@ -25,13 +25,14 @@
 
 #include <atomic>
 #include <cstdint>
+#include <deque>
 #include <functional>
-#include <map>
 #include <memory>
 #include <mutex>
 #include <optional>
 #include <set>
 #include <string>
+#include <unordered_set>
 #include <vector>
 
 #include "mmreshard.h"
@@ -180,10 +181,17 @@ class HipExecuteContext {
                    const std::vector<StoreHandle>& pipelined, const std::string& task_name);
   void OffloadHtoD(int64_t local_device_id, const std::vector<StoreHandle>& to_offload, const std::string& task_name);
 
-  void OpenWindow() {}
+  // zuku_execute_context_impl.cc:128-143: one window per execution; OpenWindow waits for the oldest window once
+  // kMaxOpenWindows (8, :46) are still running on the device, CloseWindow marks the end of this one.
+  void OpenWindow();
   void CloseWindow();
+  // :347-354.  on_done runs on a thread the context owns, once everything issued so far is done; it may use the
+  // context (drop buffers, issue work).  The call does not wait.
   void RunAfterAllTasks(int64_t local_device_id, std::function<void()> on_done);
+  // :458-460: a named mark in the profile (a roctx marker).
   void MarkProfile(const std::string& name);
+  // :462-486: named timers, any number pending, neither call waits for the device.  A second StartTimer of a running
+  // name changes nothing; StopTimer of an unknown name prints the reference's warning and returns.
   void StartTimer(const std::string& name);
   void StopTimer(const std::string& name);
   std::set<int> GetLocalDevices() { return local_devices_; }
@@ -210,32 +218,46 @@ class HipExecuteContext {
   // What ToLiteral does through SliceLocalShard (mm_pjrt_buffer.cc:84-95): blocking copy of the handle's shard.
   void CopyShardToHost(const StoreHandle& handle, void* host_dst, size_t size);
   mmr_context_stats Stats();
-  double LastTimerMilliseconds(const std::string& name);
+  // The most recent completed interval of the timer `name` (what the reference logs as "<name> finished in ...");
+  // never waits: 0 until the device has passed the first StopTimer.  *completed: intervals completed so far.
+  double LastTimerMilliseconds(const std::string& name, int64_t* completed = nullptr);
+  // The same after waiting for every stopped interval of `name` (a host wait, counted as one).
+  double WaitTimerMilliseconds(const std::string& name);
+  void SetMaxOpenWindows(int n);
 
  private:
   struct SharedStore;  // one sharded array, shared by the handles of all local devices
+  enum OpKind { kCreateStore = 0, kReshard, kOffloadDtoH, kOffloadHtoD, kNumOpKinds };
   struct ReplicatedOp {
     int64_t a{-1}, b{-1};
-    std::string what;
     std::shared_ptr<SharedStore> store;
     int arrivals{0};
   };
+  // The ops of one kind that some but not all local devices have issued, oldest first: ops[k] is call number
+  // first_seq + k of every device.
+  struct OpStream {
+    std::vector<int64_t> next_seq;  // by device position: calls so far
+    std::deque<ReplicatedOp> ops;
+    int64_t first_seq{0};
+  };
   HipExecuteContext() = default;
-  // k-th call of `kind` on this device -> the op all devices share
-  ReplicatedOp& Arrive(const char* kind, int64_t local_device_id, bool* first);
-  void Leave(const char* kind, int64_t seq, const ReplicatedOp& op);
+  // k-th call of `kind` on this device -> the op all devices share; *seq = k
+  ReplicatedOp& Arrive(OpKind kind, int64_t local_device_id, bool* first, int64_t* seq);
+  void Leave(OpKind kind);
+  void Retract(OpKind kind, int64_t local_device_id);  // the first arrival failed: it consumed no position
 
   void FlushLocked();
 
   mmr_context* ctx_{nullptr};
   bool defer_reshards_{true};
   std::vector<std::pair<std::shared_ptr<SharedStore>, std::shared_ptr<SharedStore>>> pending_;  // queued (src, dst)
+  std::unordered_set<const SharedStore*> pending_srcs_, pending_dsts_;
+  std::vector<mmr_store*> flush_srcs_, flush_dsts_;
   std::shared_ptr<std::atomic<bool>> alive_{std::make_shared<std::atomic<bool>>(true)};
   std::set<int> local_devices_;
+  std::vector<int32_t> position_of_;  // local device id -> position in local_devices_, -1 = not local
   std::mutex mu_;
-  std::map<std::string, std::map<int64_t, int64_t>> next_seq_;       // kind -> device -> calls so far
-  std::map<std::string, std::map<int64_t, ReplicatedOp>> in_flight_;  // kind -> seq -> op
-  std::map<std::string, double> timers_ms_;
+  OpStream streams_[kNumOpKinds];
   friend struct StoreHandleImpl;
 };
 
@@ -253,6 +275,8 @@ struct MpmdOperation {
 // Compute tasks are not part of it; the reshards of the whole schedule leave as one window.
 class ReshardSchedule {
  public:
+  explicit ReshardSchedule(std::string name = "reshard_schedule") : name_(std::move(name)) {}
+  const std::string& name() const { return name_; }
   Store AddStore(Store::Type type, std::string name, ShardedShape shape);
   void AddReshardTask(const Store& input, const Store& output);
   const std::vector<MpmdOperation>& schedule() const { return schedule_; }
@@ -260,10 +284,17 @@ class ReshardSchedule {
   int64_t num_roots() const { return num_roots_; }
   // parameter_stores[local device position][parameter index] -> root_stores[local device position][root index];
   // positions follow the order of ctx.GetLocalDevices().
+  // Every execution is bracketed exactly as the reference's (mm_pjrt_executable.cc:362-364 and :704-706):
+  // OpenWindow, StartTimer(name), MarkProfile("start <name>") ... StopTimer(name), CloseWindow,
+  // MarkProfile("finish <name>"); none of them waits for the device in the steady state.  on_done (optional, one
+  // per local device position) are the compute callbacks of :369-377, handed to RunAfterAllTasks as at :660-667.
   std::vector<std::vector<StoreHandle>> Execute(HipExecuteContext& ctx,
-                                                const std::vector<std::vector<StoreHandle>>& parameter_stores);
+                                                const std::vector<std::vector<StoreHandle>>& parameter_stores,
+                                                std::vector<std::function<void()>>* on_done = nullptr);
 
  private:
+  std::string name_;
+  std::string start_mark_, finish_mark_;  // "start <name>" / "finish <name>", built once
   std::vector<MpmdOperation> schedule_;
   std::set<std::pair<std::string, std::string>> already_scheduled_;
   std::vector<Store> temporaries_;

@@ -10,6 +10,12 @@ g++ -O2 -std=c++20 -Wall -Wextra -Wno-unknown-pragmas -D__HIP_PLATFORM_AMD__ -I/
   -Wl,-rpath,'$ORIGIN/../../multimesh-jax_amd' -Wl,-rpath,'$ORIGIN/../../oracle' -Wl,-rpath,/opt/rocm/lib \
   -o "${here}/hip_execute_context_test"
 echo "built ${here}/hip_execute_context_test"
+g++ -O2 -std=c++20 -Wall -Wextra -Wno-unknown-pragmas -D__HIP_PLATFORM_AMD__ -I/opt/rocm/include -I"${root}/include" \
+  -I"${root}/multimesh-jax_amd/csrc" "${here}/context_bench.cc" \
+  -L"${root}/multimesh-jax_amd" -lmmreshard -L/opt/rocm/lib -lamdhip64 \
+  -Wl,-rpath,'$ORIGIN/../../multimesh-jax_amd' -Wl,-rpath,/opt/rocm/lib \
+  -o "${here}/context_bench"
+echo "built ${here}/context_bench"
 g++ -O2 -std=c++17 -Wall -Wextra -Wno-unknown-pragmas -fPIC -shared -I"${root}/include" -I"${root}/multimesh-jax_amd/csrc" \
   "${here}/kernel_emulation.cc" -L"${root}/multimesh-jax_amd" -lmmreshard \
   -Wl,-rpath,'$ORIGIN/../../multimesh-jax_amd' -Wl,-rpath,/opt/rocm/lib \

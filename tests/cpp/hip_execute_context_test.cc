@@ -6,11 +6,13 @@
 //
 // Needs a GPU.  Prints "OK" and exits 0 on success.
 #include <atomic>
+#include <chrono>
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
 #include <stdexcept>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include <hip/hip_runtime_api.h>
@@ -110,12 +112,33 @@ static int run() {
     EXPECT(ctx->HasLocalShard(root[d]) == (d >= 8));
   }
 
-  // schedule loop: the Reshard op, issued by every local device
-  ctx->StartTimer("execute");
-  for (int d = 0; d < kLocal; ++d) ctx->Reshard(d, d, param[d], root[d]);
-  ctx->StopTimer("execute");
-  EXPECT(ctx->Stats().reshard_calls == 1);  // the copy ran once, not twelve times
-  EXPECT(ctx->Stats().plans_built == 1);
+  // schedule loop: the Reshard op, issued by every local device, inside two named timers that overlap
+  // (zuku_execute_context_impl.cc:462-486: any number pending, keyed by name, neither call waits)
+  {
+    const int64_t syncs0 = ctx->Stats().host_blocking_syncs;
+    ctx->StartTimer("execute");
+    ctx->StartTimer("execute+readback");
+    ctx->StartTimer("execute");  // already running: stays as it is (pending_timers_.emplace)
+    for (int d = 0; d < kLocal; ++d) ctx->Reshard(d, d, param[d], root[d]);
+    ctx->StopTimer("execute");
+    ctx->StopTimer("no such timer");  // a warning, as in the reference
+    EXPECT(ctx->Stats().reshard_calls == 1);  // the copy ran once, not twelve times
+    EXPECT(ctx->Stats().plans_built == 1);
+    std::vector<uint16_t> scratch(4 * 16 * 256);
+    EXPECT(ctx->Stats().host_blocking_syncs == syncs0);  // none of the timer calls waited
+    ctx->CopyShardToHost(root[8], scratch.data(), scratch.size() * 2);  // device work inside the outer timer only
+    ctx->StopTimer("execute+readback");
+    int64_t done = 0;
+    const double inner = ctx->WaitTimerMilliseconds("execute");
+    const double outer = ctx->WaitTimerMilliseconds("execute+readback");
+    EXPECT(inner > 0.0 && inner < 1000.0);
+    EXPECT(outer >= inner && outer < 1000.0);
+    EXPECT(ctx->LastTimerMilliseconds("execute", &done) == inner && done == 1);
+    EXPECT(ctx->LastTimerMilliseconds("no such timer", &done) == 0.0 && done == 0);
+    ctx->MarkProfile("after the first execution");
+    EXPECT(ctx->Stats().profile_marks == 1);
+    EXPECT(ctx->Stats().timers_resolved == 2);
+  }
 
   // expectation from the CPU restatement
   std::vector<std::vector<uint16_t>> expect(4, std::vector<uint16_t>(4 * 16 * 256, 0xDEAD));
@@ -142,6 +165,43 @@ static int run() {
     ctx->RunAfterAllTasks(0, nullptr);  // no callback: nothing to do (zuku_execute_context_impl.cc:349)
     EXPECT(mmr_sync(ctx->raw()) == MMR_OK);
     EXPECT(fired.load() == 1);
+    // The reference's callback completes a future whose continuations drop buffers (mm_pjrt_executable.cc:373-375):
+    // a callback may use the context.  This one lets go of the last handles of a store (its memory returns to the
+    // pool), creates another one and reads the context's statistics; it runs on a thread the context owns.
+    std::vector<StoreHandle> doomed(kLocal);
+    for (int d = 0; d < kLocal; ++d) doomed[d] = ctx->CreateStore(d, d, dst, {.name = "dropped by a callback"});
+    const int64_t live = ctx->Stats().stores_live;
+    std::atomic<int64_t> seen_live{-1};
+    std::atomic<bool> on_other_thread{false};
+    const std::thread::id caller = std::this_thread::get_id();
+    auto held = std::make_shared<std::vector<StoreHandle>>(std::move(doomed));
+    ctx->RunAfterAllTasks(0, [&, held]() mutable {
+      on_other_thread.store(std::this_thread::get_id() != caller);
+      for (StoreHandle& h : *held) ctx->Destroy(h);
+      seen_live.store(ctx->Stats().stores_live);
+      StoreHandle again = ctx->CreateStore(0, 0, src, {.name = "made by a callback"});
+      for (int d = 1; d < kLocal; ++d) (void)ctx->CreateStore(d, d, src, {.name = "made by a callback"});
+      (void)again;
+    });
+    held.reset();
+    EXPECT(mmr_sync(ctx->raw()) == MMR_OK);  // also waits for the callbacks whose turn has come
+    EXPECT(on_other_thread.load());
+    EXPECT(seen_live.load() == live - 1);
+    EXPECT(ctx->Stats().stores_live == live - 1);  // the callback's own store went when it returned
+  }
+  // Destroy drops one reference (zuku_execute_context_impl.cc:356-361): a copy of the handle - what a zero-copy view
+  // of the tile holds, mm_pjrt_buffer.cc:27-36 - keeps working after the buffer that made it destroyed its own
+  {
+    std::vector<StoreHandle> owner(kLocal), view(kLocal);
+    for (int d = 0; d < kLocal; ++d) owner[d] = ctx->CreateStore(d, d, dst, {.name = "viewed"});
+    for (int d = 0; d < kLocal; ++d) view[d] = owner[d];  // shares the impl
+    const int64_t live = ctx->Stats().stores_live;
+    for (int d = 0; d < kLocal; ++d) ctx->Destroy(owner[d]);
+    EXPECT(ctx->Stats().stores_live == live);
+    EXPECT(ctx->SliceLocalShard(9, view[9]) != nullptr);
+    EXPECT(ctx->HasLocalShard(view[9]) && !ctx->HasLocalShard(owner[9]));
+    for (int d = 0; d < kLocal; ++d) ctx->Destroy(view[d]);
+    EXPECT(ctx->Stats().stores_live == live - 1);
   }
   // a device outside the store's device list has no shard to slice
   EXPECT(throws([&] { ctx->SliceLocalShard(0, root[0]); }, "holds no shard"));
@@ -332,8 +392,70 @@ static int run() {
     EXPECT(steady1.device_allocations == steady0.device_allocations);
     EXPECT(steady1.bindings_built == steady0.bindings_built);
     EXPECT(steady1.plans_built == steady0.plans_built);
-    EXPECT(steady1.host_blocking_syncs == steady0.host_blocking_syncs);
+    // ... with the bracket every execution carries (OpenWindow, StartTimer, MarkProfile ... StopTimer, CloseWindow,
+    // MarkProfile): the only wait it may cause is the window limit's
+    EXPECT(steady1.host_blocking_syncs - steady1.window_waits == steady0.host_blocking_syncs - steady0.window_waits);
+    EXPECT(steady1.windows_opened - steady0.windows_opened == 5);
+    EXPECT(steady1.profile_marks - steady0.profile_marks == 10);
     EXPECT(steady1.pool_hits - steady0.pool_hits == 10);
+    int64_t timed = 0;
+    const double last = sc->WaitTimerMilliseconds(schedule.name());
+    (void)sc->LastTimerMilliseconds(schedule.name(), &timed);
+    EXPECT(timed == 9 && last > 0.0 && last < 1000.0);  // one interval per execution so far
+    // the compute callbacks of an execution (mm_pjrt_executable.cc:369-377, 660-667): one per local device
+    std::atomic<int> fired{0};
+    std::vector<std::function<void()>> on_done;
+    for (int d = 0; d < kLocal; ++d) on_done.push_back([&fired] { fired.fetch_add(1); });
+    schedule.Execute(*sc, params, &on_done);
+    EXPECT(mmr_sync(sc->raw()) == MMR_OK);
+    EXPECT(fired.load() == kLocal);
+  }
+
+  // Window back-pressure (zuku_execute_context_impl.cc:46, 128-136): with 8 windows still running on the device the
+  // ninth OpenWindow waits for the oldest, the eighth does not.  The device is held at a host function on the
+  // context's stream (no kernel waits for anything), released by this test; it lets go by itself after 20 s.
+  {
+    auto wc = HipExecuteContext::Create({0});
+    void* stream = nullptr;
+    EXPECT(mmr_context_stream(wc->raw(), &stream) == MMR_OK);
+    static std::atomic<bool> gate_open{false};
+    gate_open.store(false);
+    EXPECT(hipLaunchHostFunc(static_cast<hipStream_t>(stream),
+                             [](void*) {
+                               const auto until = std::chrono::steady_clock::now() + std::chrono::seconds(20);
+                               while (!gate_open.load() && std::chrono::steady_clock::now() < until)
+                                 std::this_thread::sleep_for(std::chrono::milliseconds(1));
+                             },
+                             nullptr) == hipSuccess);
+    const mmr_context_stats w0 = wc->Stats();
+    for (int w = 0; w < 8; ++w) {
+      wc->OpenWindow();
+      wc->CloseWindow();
+    }
+    const mmr_context_stats w1 = wc->Stats();
+    EXPECT(w1.windows_opened - w0.windows_opened == 8);
+    EXPECT(w1.window_waits == w0.window_waits && w1.host_blocking_syncs == w0.host_blocking_syncs);
+    std::atomic<bool> ninth_returned{false};
+    std::thread ninth([&] {
+      wc->OpenWindow();
+      ninth_returned.store(true);
+    });
+    std::this_thread::sleep_for(std::chrono::milliseconds(200));
+    const bool blocked = !ninth_returned.load();
+    gate_open.store(true);
+    ninth.join();
+    EXPECT(blocked);
+    wc->CloseWindow();
+    const mmr_context_stats w2 = wc->Stats();
+    EXPECT(w2.window_waits - w1.window_waits == 1);
+    EXPECT(w2.host_blocking_syncs - w1.host_blocking_syncs == 1);
+    // a higher limit: nothing waits
+    wc->SetMaxOpenWindows(64);
+    for (int w = 0; w < 20; ++w) {
+      wc->OpenWindow();
+      wc->CloseWindow();
+    }
+    EXPECT(wc->Stats().window_waits == w2.window_waits);
   }
 
   // Free(keep_in_cache) + CreateStore(allocate_from_cache) on a fresh context

@@ -367,8 +367,9 @@ def test_plan_and_binding_caches(ctx):
     ctx.Reshard(a, b)   # builds the device tables
     ctx.Reshard(a, b)   # finds them
     ctx.Reshard(c, d)   # other buffers: argument block again, same plan
-    ctx.Sync()
     s1 = ctx.stats
+    ctx.Sync()
+    assert ctx.stats["host_blocking_syncs"] == s1["host_blocking_syncs"] + 1  # a wait the caller asked for is counted
     assert s1["plans_built"] - s0["plans_built"] == 1
     assert s1["plan_cache_hits"] - s0["plan_cache_hits"] == 3
     assert s1["inline_launches"] - s0["inline_launches"] == 2
@@ -557,6 +558,12 @@ def test_reshard_replays_from_a_hip_graph():
         assert hip.hipStreamBeginCapture(stream, 0) == 0  # hipStreamCaptureModeGlobal
         with pytest.raises(mm.MmrError, match="capturing"):
             ctx.Reshard(other_srcs[0], other_dsts[0])  # not bound: would allocate
+        with pytest.raises(mm.MmrError, match="capturing") as refused:
+            ctx.ReshardBatchStatic(srcs, dsts)  # copies its tables from host memory on every call
+        assert refused.value.status_name == "INVALID_ARGUMENT"
+        for call in (lambda: ctx.StartTimer("t"), ctx.OpenWindow, ctx.CloseWindow):
+            with pytest.raises(mm.MmrError, match="capturing"):
+                call()  # events recorded into a graph could never be read back
         ctx.ReshardBatch(srcs, dsts)
         graph = C.c_void_p()
         assert hip.hipStreamEndCapture(stream, C.byref(graph)) == 0
@@ -592,6 +599,73 @@ def test_reshard_replays_from_a_hip_graph():
         assert hip.hipGraphDestroy(graph) == 0
     finally:
         ctx.close()
+
+
+def test_rotating_buffer_sets_beyond_the_binding_cache_neither_allocate_nor_wait():
+    """80 sets of buffers take turns through one plan whose tables have to live in device memory: more sets than the
+    cache of bound tables holds (64), so every launch recycles the least recently used block and uploads its tables
+    again - through the pinned staging arena, into a pooled block.  After the warm-up rounds 200 more reshards make
+    no device allocation and no host wait; a sample of the results is checked against the oracle."""
+    arrays = workloads.config(1, 16)
+    gs = [workloads.generate(a) for a in arrays]
+    with mm.ReshardContext(0) as ctx:
+        ctx.set_plan_options(0, 0, 0, B.MMR_PLAN_NO_INLINE)  # tables never travel in the argument block
+        sets = [make_stores(ctx, arrays, gs) for _ in range(80)]
+        ctx.Sync()
+        say("rotating 80 buffer sets through one plan")
+        for srcs, dsts in sets + sets[:20]:
+            ctx.ReshardBatch(srcs, dsts)
+        warm = ctx.stats
+        assert warm["bindings_cached"] == 64
+        for i in range(200):
+            srcs, dsts = sets[(20 + i) % 80]
+            ctx.ReshardBatch(srcs, dsts)
+        after = ctx.stats
+        assert after["reshard_calls"] - warm["reshard_calls"] == 200
+        assert after["bindings_built"] - warm["bindings_built"] == 200  # every one of them a miss
+        assert after["device_allocations"] == warm["device_allocations"]
+        assert after["host_blocking_syncs"] == warm["host_blocking_syncs"]
+        assert after["bindings_cached"] == 64
+        ctx.Sync()
+        for k in (0, 19, 20, 63, 64, 79):
+            _compare(arrays, gs, [read_all(ctx, d) for d in sets[k][1]])
+
+
+def test_named_timers_windows_and_marks():
+    """The per-execution bracket of the reference (OpenWindow, StartTimer, MarkProfile ... StopTimer, CloseWindow,
+    MarkProfile; mm_pjrt_executable.cc:362-364, 704-706) through the C ABI: named timers overlap and never make the
+    host wait, windows beyond the limit do."""
+    arrays = workloads.config(2, 4)
+    gs = [workloads.generate(a) for a in arrays]
+    with mm.ReshardContext(0) as ctx:
+        srcs, dsts = make_stores(ctx, arrays, gs)
+        ctx.ReshardBatch(srcs, dsts)  # plan built
+        ctx.Sync()
+        s0 = ctx.stats
+        for step in range(12):
+            ctx.OpenWindow()
+            ctx.StartTimer("step")
+            ctx.StartTimer("inner")
+            ctx.MarkProfile("start step")
+            ctx.ReshardBatch(srcs, dsts)
+            ctx.StopTimer("inner")
+            ctx.ReshardBatch(srcs, dsts)
+            ctx.StopTimer("step")
+            ctx.CloseWindow()
+            ctx.MarkProfile("finish step")
+        s1 = ctx.stats
+        # the only host waits are the window limit's (12 windows of two 2 x 32 MiB reshards, at most 8 in flight)
+        assert s1["host_blocking_syncs"] - s0["host_blocking_syncs"] == s1["window_waits"] - s0["window_waits"]
+        assert s1["windows_opened"] - s0["windows_opened"] == 12
+        assert s1["profile_marks"] - s0["profile_marks"] == 24
+        with pytest.warns(UserWarning, match="does not exist"):
+            ctx.StopTimer("never started")
+        step_ms, n_step = ctx.TimerResult("step", wait=True)
+        inner_ms, n_inner = ctx.TimerResult("inner", wait=True)
+        assert n_step == 12 and n_inner == 12
+        assert 0.0 < inner_ms < step_ms < 100.0
+        assert ctx.TimerResult("never started") == (0.0, 0)
+        _compare(arrays, gs, [read_all(ctx, d) for d in dsts])
 
 
 def test_table_order_is_tuned_on_request_and_results_do_not_change():

@@ -1,6 +1,6 @@
 """The entry point that allocates nothing (mmr_reshard_batch_static): same kernels as mmr_reshard_batch, tables in
-the GPU's static scratch array.  Checked through the C ABI against mmr_reshard_batch, bit for bit, on two calls in a
-row, the second with a smaller input."""
+the GPU's static scratch array.  Checked through the C ABI against mmr_reshard_batch and against the oracle, bit for
+bit, on two calls in a row, the second with a smaller input; and with two contexts taking turns on the one array."""
 import sys
 
 import pytest
@@ -9,7 +9,7 @@ import multimesh_jax_amd as mm
 from multimesh_jax_amd import _binding as B, workloads
 
 from gpu_helpers import make_stores, read_all
-from helpers import test_config
+from helpers import oracle_outputs, test_config
 
 pytestmark = pytest.mark.gpu
 
@@ -33,6 +33,11 @@ def _both_ways(ctx, arrays):
     after = ctx.stats
     ref = [read_all(ctx, d) for d in dsts_ref]
     got = [read_all(ctx, d) for d in dsts_static]
+    for a, g, out in zip(arrays, gs, got):  # and against the oracle, like every other GPU test
+        expect = oracle_outputs(a, g)
+        assert sorted(out) == sorted(expect)
+        for dev in expect:
+            assert out[dev].tobytes() == expect[dev].tobytes(), (a["name"], dev)
     return ref, got, before, after
 
 
@@ -76,3 +81,33 @@ def test_static_entry_point_refuses_plans_beyond_the_array():
         assert e.value.status_name == "INVALID_ARGUMENT" and "static scratch" in str(e.value)
         ctx.ReshardBatch(srcs, dsts)  # the allocating entry point takes it
         ctx.Sync()
+
+
+def test_two_contexts_take_turns_on_the_static_array():
+    """The array is one per GPU and process.  Two contexts (two streams) that call the static entry point in turn,
+    with no host synchronisation in between, are ordered on the device: each call's stream waits for the kernels of
+    the array's previous user.  Results against the oracle."""
+    a_arrays = workloads.config(2, 4)
+    b_arrays = workloads.config(5, 8)
+    a_gs = [workloads.generate(a) for a in a_arrays]
+    b_gs = [workloads.generate(a) for a in b_arrays]
+    with mm.ReshardContext(0) as ca, mm.ReshardContext(0) as cb:
+        a_sets = [make_stores(ca, a_arrays, a_gs) for _ in range(3)]
+        b_sets = [make_stores(cb, b_arrays, b_gs) for _ in range(3)]
+        ca.Sync()
+        cb.Sync()
+        say("two contexts, six interleaved static calls")
+        before = (ca.stats["host_blocking_syncs"], cb.stats["host_blocking_syncs"])
+        for k in range(3):
+            ca.ReshardBatchStatic(*a_sets[k])
+            cb.ReshardBatchStatic(*b_sets[k])
+        assert (ca.stats["host_blocking_syncs"], cb.stats["host_blocking_syncs"]) == before  # ordered on the device
+        ca.Sync()
+        cb.Sync()
+        for ctx, arrays, gs, sets in ((ca, a_arrays, a_gs, a_sets), (cb, b_arrays, b_gs, b_sets)):
+            for _, dsts in sets:
+                for a, g, d in zip(arrays, gs, dsts):
+                    expect = oracle_outputs(a, g)
+                    got = read_all(ctx, d)
+                    for dev in expect:
+                        assert got[dev].tobytes() == expect[dev].tobytes(), (a["name"], dev)
