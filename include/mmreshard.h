@@ -429,7 +429,9 @@ int mmr_sync(mmr_context* ctx);
  * mmr_timer_begin: a timer of that name that is already running is left as it is (pending_timers_.emplace, :466).
  * mmr_timer_end: MMR_NOT_FOUND if no such timer is running (the reference logs a warning and goes on, :471-474).
  * An interval is read once the device has passed its end, by whichever of these calls (or mmr_window_open) comes
- * next; mmr_timer_poll never waits: *last_milliseconds is the most recent interval of `name` that has been read
+ * next.  Marks that fall on the same point of the stream (nothing queued in between: the end of one execution's timer,
+ * its window marker, the start of the next timer) share one event, while the context owns its stream and has not
+ * handed it out through mmr_context_stream.  mmr_timer_poll never waits: *last_milliseconds is the most recent interval of `name` that has been read
  * (0 if none), *completed how many have been.  mmr_timer_wait is the blocking variant: it first waits until every
  * ended interval of `name` has been read (counted in host_blocking_syncs when it has to wait). */
 int mmr_timer_begin(mmr_context* ctx, const char* name);
@@ -495,6 +497,7 @@ typedef struct {
   int64_t windows_opened;
   int64_t window_waits;         /* mmr_window_open calls that had to wait for an older window */
   int64_t profile_marks;
+  int64_t events_recorded;      /* events the timers and windows put on the stream (points that coincide share one) */
 } mmr_context_stats;
 int mmr_context_get_stats(mmr_context* ctx, mmr_context_stats* out);
 /* Stats of the cached plan of a store pair (builds it if needed). */

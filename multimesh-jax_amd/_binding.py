@@ -99,7 +99,7 @@ class ContextStats(C.Structure):
         "reshard_calls", "bytes_allocated", "bytes_high_watermark", "stores_live", "cache_hits",
         "host_bytes_allocated", "host_bytes_high_watermark", "host_blocking_syncs", "inline_launches",
         "device_allocations", "host_cache_hits", "pool_hits", "plans_cached", "bindings_cached", "invariant_checks",
-        "operation_hash", "block_pool_hits", "timers_resolved", "windows_opened", "window_waits", "profile_marks")]
+        "operation_hash", "block_pool_hits", "timers_resolved", "windows_opened", "window_waits", "profile_marks", "events_recorded")]
 
     def as_dict(self):
         return {n: getattr(self, n) for n, _ in self._fields_}

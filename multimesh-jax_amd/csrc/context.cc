@@ -163,10 +163,19 @@ struct ProfileRange {
   bool on;
 };
 
-// A named interval whose two events are recorded and whose length nobody has read yet.
+// A point on the stream's timeline: one timing event, shared by everything that marks the same point.  The end of
+// one execution's timer, the marker of its window and the start of the next execution's timer fall on one point
+// when no work was queued in between, and an event on the stream costs the device a few microseconds of idle time.
+struct StreamPoint {
+  hipEvent_t event = nullptr;
+  int refs = 0;
+  uint64_t epoch = 0;  // mmr_context::work_epoch when it was recorded
+};
+
+// A named interval whose two points are recorded and whose length nobody has read yet.
 struct TimerInterval {
   std::string name;
-  hipEvent_t start = nullptr, stop = nullptr;
+  StreamPoint *start = nullptr, *stop = nullptr;
 };
 struct TimerResult {
   float last_ms = 0;
@@ -260,12 +269,18 @@ struct mmr_context {
   std::vector<char> fill_scratch;  // tables are assembled here, then copied into the arena
   // events are created once and reused (creating one costs a runtime lock)
   std::vector<hipEvent_t> free_plain_events, free_timing_events;
+  // Bumped by every entry point that may queue work on the stream; a StreamPoint is reused only while it is still
+  // the last thing on the stream.  Once the caller has asked for the stream (mmr_context_stream) or brought its own,
+  // work may arrive that the library does not see, and points are no longer shared.
+  std::atomic<uint64_t> work_epoch{1};
+  bool stream_exposed = false;
+  StreamPoint* last_point = nullptr;
   // named deferred timers (StartTimer / StopTimer)
-  std::unordered_map<std::string, hipEvent_t> pending_timers;
+  std::unordered_map<std::string, StreamPoint*> pending_timers;
   std::deque<TimerInterval> resolving;
   std::unordered_map<std::string, TimerResult> timer_results;
   // execution windows (OpenWindow / CloseWindow)
-  std::deque<hipEvent_t> window_markers;
+  std::deque<StreamPoint*> window_markers;
   int32_t max_open_windows = 8;
   // callbacks of mmr_context_run_after: the stream's host function only queues them here; this thread runs them
   std::thread callback_thread;
@@ -364,6 +379,38 @@ int take_event(mmr_context* ctx, bool timing, hipEvent_t* out) {
 void give_event(mmr_context* ctx, bool timing, hipEvent_t e) {
   if (e) (timing ? ctx->free_timing_events : ctx->free_plain_events).push_back(e);
 }
+
+void release_point(mmr_context* ctx, StreamPoint* p) {
+  if (!p || --p->refs > 0) return;
+  give_event(ctx, true, p->event);
+  delete p;
+}
+
+// The current end of the stream as a point the caller holds one reference to.
+int mark_point(mmr_context* ctx, StreamPoint** out) {
+  const uint64_t epoch = ctx->work_epoch.load();
+  if (ctx->last_point && ctx->last_point->epoch == epoch && ctx->owns_stream && !ctx->stream_exposed) {
+    ctx->last_point->refs += 1;
+    *out = ctx->last_point;
+    return MMR_OK;
+  }
+  auto p = std::make_unique<StreamPoint>();
+  if (int rc = take_event(ctx, true, &p->event)) return rc;
+  const hipError_t e = hipEventRecord(p->event, ctx->stream);
+  if (e != hipSuccess) {
+    give_event(ctx, true, p->event);
+    return fail(MMR_HIP_ERROR, "hipEventRecord failed: %s", hipGetErrorString(e));
+  }
+  ctx->stats.events_recorded += 1;
+  p->epoch = epoch;
+  p->refs = 2;  // the caller's and last_point's
+  release_point(ctx, ctx->last_point);
+  ctx->last_point = p.get();
+  *out = p.release();
+  return MMR_OK;
+}
+
+void note_work(mmr_context* ctx) { ctx->work_epoch.fetch_add(1); }
 
 constexpr size_t kStagingBytes = static_cast<size_t>(4) << 20;  // pinned arena of table uploads
 constexpr size_t kStagingPiece = kStagingBytes / 4;            // longer uploads go in pieces of this size
@@ -1133,7 +1180,7 @@ int resolve_timers(mmr_context* ctx, const char* wait_for) {
   if (wait_for) {
     hipEvent_t last = nullptr;
     for (const TimerInterval& t : ctx->resolving)
-      if (t.name == wait_for) last = t.stop;
+      if (t.name == wait_for) last = t.stop->event;
     if (last && hipEventQuery(last) != hipSuccess) {
       (void)hipGetLastError();
       if (int rc = blocking_wait(ctx, last)) return rc;
@@ -1141,20 +1188,20 @@ int resolve_timers(mmr_context* ctx, const char* wait_for) {
   }
   while (!ctx->resolving.empty()) {
     TimerInterval& t = ctx->resolving.front();
-    if (hipEventQuery(t.stop) != hipSuccess) {
+    if (hipEventQuery(t.stop->event) != hipSuccess) {
       (void)hipGetLastError();
       break;
     }
     float ms = 0;
-    MMR_HIP(hipEventElapsedTime(&ms, t.start, t.stop));
+    if (t.start != t.stop) MMR_HIP(hipEventElapsedTime(&ms, t.start->event, t.stop->event));
     TimerResult& r = ctx->timer_results[t.name];
     r.last_ms = ms;
     r.completed += 1;
     ctx->stats.timers_resolved += 1;
     if (ctx->flags & MMR_LOG_TIMERS)  // "<name> finished in <s>s" (zuku_execute_context_impl.cc:478-482)
       std::fprintf(stderr, "%s finished in %gs\n", t.name.c_str(), static_cast<double>(ms) * 1e-3);
-    give_event(ctx, true, t.start);
-    give_event(ctx, true, t.stop);
+    release_point(ctx, t.start);
+    release_point(ctx, t.stop);
     ctx->resolving.pop_front();
   }
   return MMR_OK;
@@ -1245,12 +1292,13 @@ void mmr_context_destroy(mmr_context* ctx) {
   if (ctx->t1) (void)hipEventDestroy(ctx->t1);
   for (hipEvent_t e : ctx->laps) (void)hipEventDestroy(e);
   for (auto& u : ctx->staged) (void)hipEventDestroy(u.consumed);
-  for (auto& t : ctx->pending_timers) (void)hipEventDestroy(t.second);
+  for (auto& t : ctx->pending_timers) release_point(ctx, t.second);
   for (auto& t : ctx->resolving) {
-    (void)hipEventDestroy(t.start);
-    (void)hipEventDestroy(t.stop);
+    release_point(ctx, t.start);
+    release_point(ctx, t.stop);
   }
-  for (hipEvent_t e : ctx->window_markers) (void)hipEventDestroy(e);
+  for (StreamPoint* p : ctx->window_markers) release_point(ctx, p);
+  release_point(ctx, ctx->last_point);  // every point's event is back in the pool now
   for (hipEvent_t e : ctx->free_plain_events) (void)hipEventDestroy(e);
   for (hipEvent_t e : ctx->free_timing_events) (void)hipEventDestroy(e);
   {  // the stream is idle: whoever uses the static array next has nothing of this context to wait for
@@ -1271,6 +1319,8 @@ void mmr_context_destroy(mmr_context* ctx) {
 
 int mmr_context_stream(mmr_context* ctx, void** hip_stream) {
   if (!ctx || !hip_stream) return fail(MMR_INVALID_ARGUMENT, "null argument");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  ctx->stream_exposed = true;  // the caller may queue work the library does not see
   *hip_stream = ctx->stream;
   return MMR_OK;
 }
@@ -1313,6 +1363,7 @@ int mmr_store_create_ex(mmr_context* ctx, const mmr_sharded_shape* shape, const 
                         int64_t min_cache_size, mmr_store** out) {
   if (!ctx || !shape || !out) return fail(MMR_INVALID_ARGUMENT, "null argument");
   std::lock_guard<std::mutex> lock(ctx->mu);
+  note_work(ctx);
   if (int rc = use_device(ctx)) return rc;
   auto s = std::make_unique<mmr_store>();
   if (int rc = mmr::make_side(*shape, &s->side)) return rc;
@@ -1451,6 +1502,7 @@ int mmr_store_assemble(mmr_context* ctx, mmr_store* store, int64_t device, const
                        int32_t data_on_device) {
   if (!ctx) return fail(MMR_INVALID_ARGUMENT, "null context");
   std::lock_guard<std::mutex> lock(ctx->mu);
+  note_work(ctx);
   if (int rc = check_store(ctx, store, "assembled")) return rc;
   int64_t k = 0;
   if (int rc = tile_index(store, device, &k)) return rc;
@@ -1516,6 +1568,7 @@ int mmr_store_shard_ptr(mmr_context* ctx, mmr_store* store, int64_t device, void
 int mmr_store_read_shard(mmr_context* ctx, mmr_store* store, int64_t device, void* host_dst, size_t size) {
   if (!ctx || !host_dst) return fail(MMR_INVALID_ARGUMENT, "null argument");
   std::lock_guard<std::mutex> lock(ctx->mu);
+  note_work(ctx);
   if (int rc = check_store(ctx, store, "read")) return rc;
   int64_t k = 0;
   if (int rc = tile_index(store, device, &k)) return rc;
@@ -1578,6 +1631,7 @@ int mmr_store_adopt(mmr_context* ctx, const mmr_sharded_shape* shape, const char
 int mmr_store_offload(mmr_context* ctx, mmr_store* store) {
   if (!ctx) return fail(MMR_INVALID_ARGUMENT, "null context");
   std::lock_guard<std::mutex> lock(ctx->mu);
+  note_work(ctx);
   if (int rc = check_store(ctx, store, "offloaded")) return rc;
   if (store->offloaded()) return MMR_OK;
   if (!store->adopted.empty()) return fail(MMR_INVALID_ARGUMENT, "store %lld lives in caller-owned buffers", (long long)store->id);
@@ -1607,6 +1661,7 @@ int mmr_store_offload(mmr_context* ctx, mmr_store* store) {
 int mmr_store_reload(mmr_context* ctx, mmr_store* store) {
   if (!ctx) return fail(MMR_INVALID_ARGUMENT, "null context");
   std::lock_guard<std::mutex> lock(ctx->mu);
+  note_work(ctx);
   if (int rc = check_store(ctx, store, "reloaded")) return rc;
   if (!store->offloaded()) return MMR_OK;
   if (int rc = use_device(ctx)) return rc;
@@ -1638,6 +1693,7 @@ int mmr_context_prepare(mmr_context* ctx, const mmr_sharded_shape* srcs, const m
   if (!ctx || n < 0 || (n > 0 && (!srcs || !dsts))) return fail(MMR_INVALID_ARGUMENT, "bad arguments");
   if (n == 0) return MMR_OK;
   std::lock_guard<std::mutex> lock(ctx->mu);
+  note_work(ctx);
   if (int rc = use_device(ctx)) return rc;
   std::vector<mmr_sharded_shape> s(srcs, srcs + n), d(dsts, dsts + n);
   DevicePlan* dp = nullptr;
@@ -1646,6 +1702,7 @@ int mmr_context_prepare(mmr_context* ctx, const mmr_sharded_shape* srcs, const m
 
 int mmr_context_wait_event(mmr_context* ctx, void* hip_event) {
   if (!ctx || !hip_event) return fail(MMR_INVALID_ARGUMENT, "null argument");
+  note_work(ctx);
   MMR_HIP(hipStreamWaitEvent(ctx->stream, static_cast<hipEvent_t>(hip_event), 0));
   return MMR_OK;
 }
@@ -1659,24 +1716,28 @@ int mmr_context_record_event(mmr_context* ctx, void* hip_event) {
 int mmr_reshard(mmr_context* ctx, mmr_store* src, mmr_store* dst) {
   if (!ctx) return fail(MMR_INVALID_ARGUMENT, "null context");
   std::lock_guard<std::mutex> lock(ctx->mu);
+  note_work(ctx);
   return reshard_locked(ctx, &src, &dst, 1);
 }
 
 int mmr_reshard_batch(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int32_t n) {
   if (!ctx || n < 0 || (n > 0 && (!srcs || !dsts))) return fail(MMR_INVALID_ARGUMENT, "bad batch arguments");
   std::lock_guard<std::mutex> lock(ctx->mu);
+  note_work(ctx);
   return reshard_locked(ctx, srcs, dsts, n);
 }
 
 int mmr_reshard_batch_static(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int32_t n) {
   if (!ctx || n < 0 || (n > 0 && (!srcs || !dsts))) return fail(MMR_INVALID_ARGUMENT, "bad batch arguments");
   std::lock_guard<std::mutex> lock(ctx->mu);
+  note_work(ctx);
   return reshard_static_locked(ctx, srcs, dsts, n);
 }
 
 int mmr_reshard_tune(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int32_t n, int64_t* order_used) {
   if (!ctx || n <= 0 || !srcs || !dsts) return fail(MMR_INVALID_ARGUMENT, "bad batch arguments");
   std::lock_guard<std::mutex> lock(ctx->mu);
+  note_work(ctx);
   return tune_locked(ctx, srcs, dsts, n, order_used);
 }
 
@@ -1704,12 +1765,14 @@ int mmr_reshard_validate(mmr_context* ctx, mmr_store* src, mmr_store* dst) {
 int mmr_reshard_bind(mmr_context* ctx, mmr_store* const* srcs, mmr_store* const* dsts, int32_t n) {
   if (!ctx || n < 0 || (n > 0 && (!srcs || !dsts))) return fail(MMR_INVALID_ARGUMENT, "bad batch arguments");
   std::lock_guard<std::mutex> lock(ctx->mu);
+  note_work(ctx);
   return reshard_locked(ctx, srcs, dsts, n, /*launch=*/false);
 }
 
 int mmr_context_run_after(mmr_context* ctx, void (*fn)(void*), void* arg) {
   if (!ctx || !fn) return fail(MMR_INVALID_ARGUMENT, "null argument");
   MMR_HIP(hipSetDevice(ctx->device));
+  note_work(ctx);
   {
     std::lock_guard<std::mutex> lock(ctx->callback_mu);
     if (!ctx->callback_thread.joinable()) ctx->callback_thread = std::thread(callback_loop, ctx);
@@ -1796,13 +1859,8 @@ int mmr_timer_begin(mmr_context* ctx, const char* name) {
   if (int rc = resolve_timers(ctx, nullptr)) return rc;
   // pending_timers_.emplace(name, ...) (zuku_execute_context_impl.cc:466): a timer of that name already running stays
   if (ctx->pending_timers.count(name)) return MMR_OK;
-  hipEvent_t start = nullptr;
-  if (int rc = take_event(ctx, true, &start)) return rc;
-  const hipError_t e = hipEventRecord(start, ctx->stream);
-  if (e != hipSuccess) {
-    give_event(ctx, true, start);
-    return fail(MMR_HIP_ERROR, "hipEventRecord failed: %s", hipGetErrorString(e));
-  }
+  StreamPoint* start = nullptr;
+  if (int rc = mark_point(ctx, &start)) return rc;
   ctx->pending_timers.emplace(name, start);
   return MMR_OK;
 }
@@ -1818,12 +1876,7 @@ int mmr_timer_end(mmr_context* ctx, const char* name) {
   TimerInterval t;
   t.name = it->first;
   t.start = it->second;
-  if (int rc = take_event(ctx, true, &t.stop)) return rc;
-  const hipError_t e = hipEventRecord(t.stop, ctx->stream);
-  if (e != hipSuccess) {
-    give_event(ctx, true, t.stop);
-    return fail(MMR_HIP_ERROR, "hipEventRecord failed: %s", hipGetErrorString(e));
-  }
+  if (int rc = mark_point(ctx, &t.stop)) return rc;
   ctx->pending_timers.erase(it);
   ctx->resolving.push_back(std::move(t));
   return resolve_timers(ctx, nullptr);
@@ -1880,19 +1933,19 @@ int mmr_window_open(mmr_context* ctx) {
   if (int rc = use_device(ctx)) return rc;
   if (int rc = refuse_capture(ctx, "mmr_window_open")) return rc;
   // windows the device has finished are no longer in flight
-  while (!ctx->window_markers.empty() && hipEventQuery(ctx->window_markers.front()) == hipSuccess) {
-    give_event(ctx, false, ctx->window_markers.front());
+  while (!ctx->window_markers.empty() && hipEventQuery(ctx->window_markers.front()->event) == hipSuccess) {
+    release_point(ctx, ctx->window_markers.front());
     ctx->window_markers.pop_front();
   }
   (void)hipGetLastError();  // hipErrorNotReady of the query that ended the loop
   // "we have to limit the maximum number of open windows" (zuku_execute_context_impl.cc:128-136): the caller waits
   // for the oldest window while max_open_windows are still running
   while (static_cast<int64_t>(ctx->window_markers.size()) >= ctx->max_open_windows) {
-    hipEvent_t oldest = ctx->window_markers.front();
+    StreamPoint* oldest = ctx->window_markers.front();
     ctx->window_markers.pop_front();
     ctx->stats.window_waits += 1;
-    const int rc = blocking_wait(ctx, oldest);
-    give_event(ctx, false, oldest);
+    const int rc = blocking_wait(ctx, oldest->event);
+    release_point(ctx, oldest);
     if (rc != MMR_OK) return rc;
   }
   ctx->stats.windows_opened += 1;
@@ -1904,13 +1957,8 @@ int mmr_window_close(mmr_context* ctx) {
   std::lock_guard<std::mutex> lock(ctx->mu);
   if (int rc = use_device(ctx)) return rc;
   if (int rc = refuse_capture(ctx, "mmr_window_close")) return rc;
-  hipEvent_t marker = nullptr;  // merge_events(last_execute_events_) (:139): everything queued so far
-  if (int rc = take_event(ctx, false, &marker)) return rc;
-  const hipError_t e = hipEventRecord(marker, ctx->stream);
-  if (e != hipSuccess) {
-    give_event(ctx, false, marker);
-    return fail(MMR_HIP_ERROR, "hipEventRecord failed: %s", hipGetErrorString(e));
-  }
+  StreamPoint* marker = nullptr;  // merge_events(last_execute_events_) (:139): everything queued so far
+  if (int rc = mark_point(ctx, &marker)) return rc;
   ctx->window_markers.push_back(marker);
   return MMR_OK;
 }

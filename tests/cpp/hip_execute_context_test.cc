@@ -397,6 +397,8 @@ static int run() {
     EXPECT(steady1.host_blocking_syncs - steady1.window_waits == steady0.host_blocking_syncs - steady0.window_waits);
     EXPECT(steady1.windows_opened - steady0.windows_opened == 5);
     EXPECT(steady1.profile_marks - steady0.profile_marks == 10);
+    // StopTimer, CloseWindow and the next execution's StartTimer mark the same point of the stream: one event
+    EXPECT(steady1.events_recorded - steady0.events_recorded == 5);
     EXPECT(steady1.pool_hits - steady0.pool_hits == 10);
     int64_t timed = 0;
     const double last = sc->WaitTimerMilliseconds(schedule.name());
