@@ -10,6 +10,7 @@
 // A memory policy `M` provides
 //   typedef ... cptr;  typedef ... ptr;          byte pointers (const / mutable)
 //   static V16 load16(cptr), load16u(cptr);       16-byte load, aligned / any alignment
+//   static V16 load16u_keep(cptr);                the same for bytes other workgroups read too (no streaming hint)
 //   static void store16(ptr, V16);                16-byte aligned store
 //   static T loadu<T>(cptr); static void storeu<T>(ptr, T);   1/2/4/8-byte, any alignment
 //   static uintptr_t addr(ptr), caddr(cptr);      numeric address (for alignment math)

@@ -425,18 +425,44 @@ MMR_HD void span_gather(const SpanGroup& g, const SpanMember& m, const SpanPiece
 // destination vector and works out its source address lane by lane, some 150 vector instructions per 16 bytes.  Here
 // the (row, piece) pairs that touch the span - its SEGMENTS, at most one per lane - are worked out once, lane s
 // taking segment s, and left in LDS as 16-byte records; an item then needs one division for its row, a few compares
-// for its piece, one LDS read and an add.  That halves the kernel's vector and scalar instruction counts (counters);
-// its time on ragged rows stayed the same, since the wait for the gathered loads is what fills it.
+// for its piece, one LDS read and an add.
+//
+// Items of a span in table mode:
+//   A  one per aligned destination vector of the span, belonging to the segment the vector's first in-span byte
+//      lies in: the 16 source bytes that start where that byte comes from (an unaligned load); if the piece row ends
+//      before the vector does, the load slides back to end with the row.
+//   B  one per segment: the first 16 bytes of the piece row (what a vector that began in the previous segment
+//      could not bring).
+// Two variations are kept as build options.  Both do what they were made for and neither makes the kernel faster
+// (3-way -> 5-way rows of 4,099 bytes on MI355X: 20.4 us as shipped, 20.8-21.4 us with either or both):
+//   MMR_SPAN_ALIGNED_LOADS  A items load the ALIGNED 16-byte vector of the source that holds their first byte
+//      (clamped to the piece row; all A items of a segment are shifted by the same amount, so they tile its
+//      middle), and a third kind of item, C, brings the last 16 bytes of the piece row or of its part inside the
+//      span.  A third fewer accesses in the vector L1 (3.19 M against 4.77 M per launch).
+//   MMR_SPAN_KEEP_EDGES  loads that touch the first or the last 128-byte line of their piece row - the lines that
+//      also hold bytes of the neighbouring piece, which the span of the neighbouring destination tile reads at
+//      about the same time - go through the caches in the ordinary way (M::load16u_keep), everything in between
+//      keeps the streaming hint.  Memory reads fall from 1.085 x to 1.013 x the source bytes.
+#ifndef MMR_SPAN_ALIGNED_LOADS
+#define MMR_SPAN_ALIGNED_LOADS 0
+#endif
+#ifndef MMR_SPAN_KEEP_EDGES
+#define MMR_SPAN_KEEP_EDGES 0
+#endif
+constexpr bool kSpanAlignedLoads = MMR_SPAN_ALIGNED_LOADS != 0;
+constexpr bool kSpanKeepEdges = MMR_SPAN_KEEP_EDGES != 0;
+
 struct SpanSegment {   // 16 bytes in LDS
   uint32_t d_lo, d_hi;  // (address of the piece row's first byte) - start, so that destination position y reads at d + y
-  uint32_t flags;       // 0: load; 1: the piece is a pad (zeros); 2: narrower than 16 bytes (gathered byte by byte)
+  uint32_t w_flags;     // bits 0-29: bytes of the piece row; bits 30-31: 0 load, 1 the piece is a pad (zeros),
+                        // 2 narrower than 16 bytes (gathered byte by byte)
   int32_t end16;        // start + w - 16: the last position a 16-byte vector of this piece row may begin at
 };
-// The item of kind B a lane brings from span_table_build to span_table_gather (the first 16 bytes of its segment).
+// The items of kind B and C a lane brings from span_table_build to span_table_gather.
 template <class M>
-struct SpanRowStart {
-  typename M::cptr from;
-  uint32_t at;
+struct SpanRowEnds {
+  typename M::cptr from_b, from_c;
+  uint32_t at_b, at_c;
   bool on, zero;
 };
 
@@ -448,9 +474,9 @@ MMR_HD SpanPieces4 span_pieces4(const SpanPiece* pc, uint32_t k) {
 }
 
 template <class M, class L, int LANES>
-MMR_HD SpanRowStart<M> span_table_build(const SpanGroup& g, const SpanMember& m, const SpanPieces4& pcs,
-                                        typename M::cptr safe, uint64_t x0, uint32_t len, uint32_t a, uint8_t* table,
-                                        uint32_t lane) {
+MMR_HD SpanRowEnds<M> span_table_build(const SpanGroup& g, const SpanMember& m, const SpanPieces4& pcs,
+                                       typename M::cptr safe, uint64_t x0, uint32_t len, uint32_t a, uint8_t* table,
+                                       uint32_t lane) {
   const uint32_t W = g.W;
   const uint64_t row0 = x0 < (1ull << 31) ? fdiv(static_cast<uint32_t>(x0), g.div_W) : x0 / W;
   const uint32_t o0 = static_cast<uint32_t>(x0 - row0 * W);
@@ -475,33 +501,42 @@ MMR_HD SpanRowStart<M> span_table_build(const SpanGroup& g, const SpanMember& m,
   const uint64_t d = src_row - static_cast<uint64_t>(static_cast<int64_t>(start));
   seg.d_lo = static_cast<uint32_t>(d);
   seg.d_hi = static_cast<uint32_t>(d >> 32);
-  seg.flags = !wide ? 2u : (fill ? 1u : 0u);
+  seg.w_flags = pk.w | ((!wide ? 2u : (fill ? 1u : 0u)) << 30);  // planner: w <= kSpanMaxRowBytes < 2^30
   seg.end16 = wide ? start + static_cast<int32_t>(pk.w) - 16 : -16;  // narrow: its vectors land in the spare bytes
-  if (on) L::store16u(table + (s << 4), V16{seg.d_lo, seg.d_hi, seg.flags, static_cast<uint32_t>(seg.end16)});
-  SpanRowStart<M> b;
+  if (on) L::store16u(table + (s << 4), V16{seg.d_lo, seg.d_hi, seg.w_flags, static_cast<uint32_t>(seg.end16)});
+  SpanRowEnds<M> b;
   b.on = on && wide;
   b.zero = fill;
-  b.from = b.on && !fill ? reinterpret_cast<typename M::cptr>(src_row) : safe;
-  int32_t drel = start < -16 ? -16 : (start > ilen ? ilen : start);  // outside the span: into the spare bytes
-  b.at = static_cast<uint32_t>(static_cast<int32_t>(16 + a) + drel);
+  const bool loads = b.on && !fill;
+  // C begins where the piece row's last 16 bytes do, or the span's if the row runs on, and never before the row
+  int32_t c = seg.end16 < ilen - 16 ? seg.end16 : ilen - 16;
+  c = c < start ? start : c;
+  b.from_b = loads ? reinterpret_cast<typename M::cptr>(src_row) : safe;
+  b.from_c = loads ? reinterpret_cast<typename M::cptr>(src_row + static_cast<uint64_t>(static_cast<int64_t>(c - start))) : safe;
+  // outside the span: into the spare bytes around it
+  const int32_t drel_b = start < -16 ? -16 : (start > ilen ? ilen : start);
+  const int32_t drel_c = c < -16 ? -16 : (c > ilen ? ilen : c);
+  b.at_b = static_cast<uint32_t>(static_cast<int32_t>(16 + a) + drel_b);
+  b.at_c = static_cast<uint32_t>(static_cast<int32_t>(16 + a) + drel_c);
   return b;
 }
 
 template <class M, class L, int LANES, int DEPTH>
 MMR_HD void span_table_gather(const SpanGroup& g, const SpanMember& m, const SpanPiece* pc, const SpanPieces4& pcs,
                               typename M::cptr safe, uint64_t x0, uint32_t len, uint32_t a, uint8_t* lds,
-                              const uint8_t* table, const SpanRowStart<M>& b, uint32_t lane) {
+                              const uint8_t* table, const SpanRowEnds<M>& b, uint32_t lane) {
   const uint32_t W = g.W;
   const uint64_t row0 = x0 < (1ull << 31) ? fdiv(static_cast<uint32_t>(x0), g.div_W) : x0 / W;
   const uint32_t o0 = static_cast<uint32_t>(x0 - row0 * W);
   const uint32_t k = m.k;
   const uint32_t n_a = (len + a + 15) >> 4;  // aligned destination vectors that overlap the span
+  constexpr int ITEMS = DEPTH + (kSpanAlignedLoads ? 2 : 1);
   // one pass unless the span is a full one in a buffer that is not 16-byte aligned (one vector more than LANES * DEPTH)
   for (uint32_t base = 0; base < n_a; base += LANES * DEPTH) {
-    V16 v[DEPTH + 1];
-    uint32_t at[DEPTH + 1];
-    bool live[DEPTH + 1], zero[DEPTH + 1];
-    typename M::cptr from[DEPTH + 1];
+    V16 v[ITEMS];
+    uint32_t at[ITEMS];
+    bool live[ITEMS], zero[ITEMS], keep[ITEMS];
+    typename M::cptr from[ITEMS];
 #pragma unroll
     for (int u = 0; u < DEPTH; ++u) {
       const uint32_t i = base + lane + u * LANES;
@@ -515,20 +550,42 @@ MMR_HD void span_table_gather(const SpanGroup& g, const SpanMember& m, const Spa
       if (k > 3) p += col >= pcs.c3.col ? 1u : 0u;
       const V16 rec = L::load16(table + ((rr * k + p) << 4));
       const int32_t end16 = static_cast<int32_t>(rec.w);
-      const int32_t yy = static_cast<int32_t>(y) < end16 ? static_cast<int32_t>(y) : end16;  // slides back to end with the piece
+      const uint32_t w = rec.z & 0x3fffffffu;
+      const int32_t start = end16 + 16 - static_cast<int32_t>(w);
+      int32_t yy = static_cast<int32_t>(y);
+      if (kSpanAlignedLoads) {
+        yy -= static_cast<int32_t>((rec.x + y) & 15u);  // back to the 16-byte boundary of the source
+        yy = yy < start ? start : yy;                   // ... but not before the piece row begins
+      }
+      yy = yy < end16 ? yy : end16;  // slides back to end with the piece row
       const uint64_t d = (static_cast<uint64_t>(rec.y) << 32) | rec.x;
-      zero[u] = rec.z != 0;
+      zero[u] = (rec.z >> 30) != 0;
       from[u] = live[u] && !zero[u] ? reinterpret_cast<typename M::cptr>(d + static_cast<uint64_t>(static_cast<int64_t>(yy))) : safe;
       at[u] = static_cast<uint32_t>(static_cast<int32_t>(16 + a) + yy);
+      // first or last 128-byte line of the piece row (low address bits suffice: the row is shorter than 4 GiB)
+      const uint32_t row_lo = rec.x + static_cast<uint32_t>(start), lo = rec.x + static_cast<uint32_t>(yy);
+      keep[u] = (lo >> 7) == (row_lo >> 7) || ((lo + 15u) >> 7) == ((row_lo + w - 1u) >> 7);
     }
     live[DEPTH] = b.on && base == 0;
     zero[DEPTH] = b.zero;
-    from[DEPTH] = base == 0 ? b.from : safe;
-    at[DEPTH] = b.at;
+    from[DEPTH] = base == 0 ? b.from_b : safe;
+    at[DEPTH] = b.at_b;
+    keep[DEPTH] = true;
+    if (kSpanAlignedLoads) {
+      live[DEPTH + 1] = live[DEPTH];
+      zero[DEPTH + 1] = b.zero;
+      from[DEPTH + 1] = base == 0 ? b.from_c : safe;
+      at[DEPTH + 1] = b.at_c;
+      keep[DEPTH + 1] = true;
+    }
 #pragma unroll
-    for (int u = 0; u <= DEPTH; ++u) v[u] = M::load16u(from[u]);
+    for (int u = 0; u < ITEMS; ++u) {
+      if (kSpanKeepEdges && u >= DEPTH) v[u] = M::load16u_keep(from[u]);
+      else if (kSpanKeepEdges) v[u] = keep[u] ? M::load16u_keep(from[u]) : M::load16u(from[u]);
+      else v[u] = M::load16u(from[u]);
+    }
 #pragma unroll
-    for (int u = 0; u <= DEPTH; ++u)
+    for (int u = 0; u < ITEMS; ++u)
       if (live[u]) L::store16u(lds + at[u], zero[u] ? V16{0, 0, 0, 0} : v[u]);
   }
   if (m.narrow) {

@@ -60,6 +60,11 @@ struct DeviceMem {
 
   static __device__ __forceinline__ V16 load16(cptr p) { return pack(ld<u32x4, 16>(p)); }
   static __device__ __forceinline__ V16 load16u(cptr p) { return pack(ld<u32x4, 1>(p)); }
+  // 16 bytes at any alignment that other workgroups read too: an ordinary cacheable load whatever NTL says
+  static __device__ __forceinline__ V16 load16u_keep(cptr p) {
+    typedef MMR_GLOBAL const u32x4 __attribute__((aligned(1))) gt;
+    return pack(*reinterpret_cast<gt*>(p));
+  }
   static __device__ __forceinline__ void store16(ptr p, V16 v) { st<u32x4, 16>(p, unpack(v)); }
   template <typename T>
   static __device__ __forceinline__ T loadu(cptr p) {
@@ -156,7 +161,7 @@ __device__ __forceinline__ void span_chunk(const SpanGroup* __restrict__ groups,
     const SpanPiece* pc = pieces + m.first_piece;
     const SpanPieces4 pcs = span_pieces4(pc, m.k);
     uint8_t* table = lds + kSpanStageBytes;
-    const SpanRowStart<M> b = span_table_build<M, DeviceLds, THREADS>(g, m, pcs, safe, x0, len, a, table, threadIdx.x);
+    const SpanRowEnds<M> b = span_table_build<M, DeviceLds, THREADS>(g, m, pcs, safe, x0, len, a, table, threadIdx.x);
     __syncthreads();
     span_table_gather<M, DeviceLds, THREADS, UNROLL>(g, m, pc, pcs, safe, x0, len, a, lds, table, b, threadIdx.x);
   } else {

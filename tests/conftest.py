@@ -40,6 +40,7 @@ def pytest_configure(config):
     # the sanitizer binary is host-only and does not travel to a GPU box: a GPU-only run does not ask for it
     gpu_only = config.getoption("markexpr", "").strip() == "gpu"
     if (_stale("tests/cpp/libmmr_emulation.so", cpp) or _stale("tests/cpp/hip_execute_context_test", cpp)
+            or _stale("tests/cpp/libmmr_emulation_span_options.so", cpp)
             or _stale("tests/cpp/context_bench", cpp)
             or (not gpu_only and _stale("tests/cpp/sanitize_sweep", cpp))) and (have_hipcc or not os.path.exists(
                 os.path.join(ROOT, "tests", "cpp", "libmmr_emulation.so"))):

@@ -21,6 +21,13 @@ g++ -O2 -std=c++17 -Wall -Wextra -Wno-unknown-pragmas -fPIC -shared -I"${root}/i
   -Wl,-rpath,'$ORIGIN/../../multimesh-jax_amd' -Wl,-rpath,/opt/rocm/lib \
   -o "${here}/libmmr_emulation.so"
 echo "built ${here}/libmmr_emulation.so"
+# the same with the span kernel's two optional variations (source-aligned loads, cacheable edge lines) switched on
+g++ -O2 -std=c++17 -Wall -Wextra -Wno-unknown-pragmas -fPIC -shared -DMMR_SPAN_ALIGNED_LOADS=1 -DMMR_SPAN_KEEP_EDGES=1 \
+  -I"${root}/include" -I"${root}/multimesh-jax_amd/csrc" \
+  "${here}/kernel_emulation.cc" -L"${root}/multimesh-jax_amd" -lmmreshard \
+  -Wl,-rpath,'$ORIGIN/../../multimesh-jax_amd' -Wl,-rpath,/opt/rocm/lib \
+  -o "${here}/libmmr_emulation_span_options.so"
+echo "built ${here}/libmmr_emulation_span_options.so"
 # Host-only sanitizer build: planner + descriptor geometry + the emulation of the kernels + a random sweep.
 g++ -O1 -g -std=c++17 -fsanitize=address,undefined -fno-sanitize-recover=undefined -fno-omit-frame-pointer \
   -Wall -Wextra -Wno-unknown-pragmas -I"${root}/include" -I"${root}/multimesh-jax_amd/csrc" \

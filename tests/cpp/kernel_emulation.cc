@@ -69,6 +69,7 @@ struct HostMem {
   }
   static mmr::V16 load16(cptr p) { return get<mmr::V16>(p, 16, "out-of-bounds load"); }
   static mmr::V16 load16u(cptr p) { return get<mmr::V16>(p, 1, "out-of-bounds load"); }
+  static mmr::V16 load16u_keep(cptr p) { return get<mmr::V16>(p, 1, "out-of-bounds load"); }
   static void store16(ptr p, mmr::V16 v) { put<mmr::V16>(p, v, 16, "out-of-bounds store"); }
   template <typename T>
   static T loadu(cptr p) { return get<T>(p, 1, "out-of-bounds load"); }
@@ -272,7 +273,7 @@ int mmr_emulate_plan(const mmr_plan* plan, void* const* slot_ptrs, const size_t*
       auto with_table = [&](auto lanes_c, auto depth_c) {
         constexpr int LANES = decltype(lanes_c)::value, DEPTH = decltype(depth_c)::value;
         const mmr::SpanPieces4 pcs = mmr::span_pieces4(pc, m.k);
-        std::vector<mmr::SpanRowStart<HostMem>> starts(LANES);
+        std::vector<mmr::SpanRowEnds<HostMem>> starts(LANES);
         for (uint32_t tid = 0; tid < LANES; ++tid)
           starts[tid] = mmr::span_table_build<HostMem, HostLds, LANES>(g, m, pcs, safe, x0, len, a, table, tid);
         for (uint32_t tid = 0; tid < LANES; ++tid)

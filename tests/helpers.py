@@ -83,18 +83,18 @@ def apply_plan(plan: "mm.Plan", buffers: Sequence[np.ndarray]) -> None:
                     dst[do:do + it] = src[so:so + it]
 
 
-_emu = None
+_emu = {}
+EMULATION_VARIANT = ""  # "_span_options": the build with the span kernel's two optional variations switched on
 
 
 def emulation_lib():
     """tests/cpp/libmmr_emulation.so: the kernels' own per-chunk code compiled for the host with bounds checks."""
-    global _emu
-    if _emu is None:
+    if EMULATION_VARIANT not in _emu:
         import ctypes as C
         import os
         import subprocess
         here = os.path.dirname(os.path.abspath(__file__))
-        path = os.path.join(here, "cpp", "libmmr_emulation.so")
+        path = os.path.join(here, "cpp", "libmmr_emulation%s.so" % EMULATION_VARIANT)
         if not os.path.exists(path):
             subprocess.check_call(["bash", os.path.join(here, "cpp", "build.sh")])
         lib = C.CDLL(path)
@@ -102,8 +102,8 @@ def emulation_lib():
         lib.mmr_emulate_plan.argtypes = [C.c_void_p, C.POINTER(C.c_void_p), C.POINTER(C.c_size_t), C.c_int64,
                                          C.c_uint32, C.c_int, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64),
                                          C.c_char_p, C.c_size_t]
-        _emu = lib
-    return _emu
+        _emu[EMULATION_VARIANT] = lib
+    return _emu[EMULATION_VARIANT]
 
 
 def _aligned_copy(buf: np.ndarray) -> np.ndarray:

@@ -28,6 +28,21 @@ def test_configs_through_the_kernel_code(index, scale, shape):
     _check(arrays, gs, shape=shape)
 
 
+def test_span_kernel_build_options_through_the_kernel_code():
+    """The span kernel's two optional variations (MMR_SPAN_ALIGNED_LOADS, MMR_SPAN_KEEP_EDGES: not in the shipped
+    build, they do not pay) keep passing the same checks on the ragged configurations."""
+    import helpers
+    helpers.EMULATION_VARIANT = "_span_options"
+    try:
+        for index, scale in ((5, 32), (6, 32), (7, 32), (8, 32), (11, 64)):
+            arrays = test_config(index, scale)
+            gs = [workloads.generate(a) for a in arrays]
+            for shape in (0, 1):
+                _check(arrays, gs, shape=shape)
+    finally:
+        helpers.EMULATION_VARIANT = ""
+
+
 @pytest.mark.parametrize("xcd_mode", [1, 2, 16, 64, 1024])
 def test_every_workgroup_mapping_visits_each_chunk_once(xcd_mode):
     for index, scale in ((2, 32), (5, 64), (4, 64)):
@@ -81,6 +96,24 @@ def ragged_2d(draw):
             "seed": 0, "dist": "raw"}
 
 
+@given(ragged_2d(), st.sampled_from([0, 1]))
+@settings(max_examples=150, deadline=None)
+def test_span_kernel_build_options_ragged_rows(a, shape):
+    import helpers
+    from oracle import reshard_oracle as ro
+    item = ro.ITEMSIZE[a["type"]]
+    rng = np.random.Generator(np.random.PCG64(29))
+    g = rng.integers(0, 256, size=int(np.prod(a["shape"])) * item, dtype=np.uint8).view(
+        ro.raw_dtype(a["type"])).reshape(a["shape"])
+    if a["shape"][1] == 1 and (a["src"]["dims"][1][1] > 1 or a["dst"]["dims"][1][1] > 1):
+        return  # trailing {1, R} would read as a replication entry
+    helpers.EMULATION_VARIANT = "_span_options"
+    try:
+        _check([a], [g], shape=shape)
+    finally:
+        helpers.EMULATION_VARIANT = ""
+
+
 @given(ragged_2d(), st.sampled_from([0, 512, 4096]), st.sampled_from([0, 1, 2, 3]))
 @settings(max_examples=150, deadline=None)
 def test_ragged_rows_through_the_kernel_code(a, chunk_bytes, shape):
@@ -108,6 +141,22 @@ def ragged_3d(draw):
             "dst": {"dims": [(outer, od, 1), (inner, 1, 2), (cols, st_dst, 0)], "dev_start": 20,
                     "dev_count": od * st_dst},
             "seed": 0, "dist": "raw"}
+
+
+@given(ragged_3d(), st.sampled_from([0, 1]))
+@settings(max_examples=120, deadline=None)
+def test_span_kernel_build_options_long_ragged_rows(a, shape):
+    import helpers
+    from oracle import reshard_oracle as ro
+    item = ro.ITEMSIZE[a["type"]]
+    rng = np.random.Generator(np.random.PCG64(31))
+    g = rng.integers(0, 256, size=int(np.prod(a["shape"])) * item, dtype=np.uint8).view(
+        ro.raw_dtype(a["type"])).reshape(a["shape"])
+    helpers.EMULATION_VARIANT = "_span_options"
+    try:
+        _check([a], [g], shape=shape)
+    finally:
+        helpers.EMULATION_VARIANT = ""
 
 
 @given(ragged_3d(), st.sampled_from([0, 512, 4096]), st.sampled_from([0, 1, 2, 3]))
