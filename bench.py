@@ -149,53 +149,69 @@ def measure(ctx, mm, workloads, args, config):
         else:
             ctx.ReshardBatch(srcs, dsts)
 
-    # Schedule-build time work (MpmdScheduler::AddReshardTask in the reference): plan, optional timing of launch
-    # orders on the first set, device tables for every set.  None of it is in the timed region.
+    # Schedule-build time work (MpmdScheduler::AddReshardTask in the reference): plan and device tables for every
+    # set.  None of it is in a timed region.
     before = ctx.stats
     step(0)
     ctx.Sync()
     launches = ctx.stats["kernel_launches"] - before["kernel_launches"]
     checked = check_parity(ctx, arrays, gs, sets[0][1], sample_only=alg_bytes > (2 << 30))
+
+    def bind_all():
+        if not args.unbatched:
+            for srcs, dsts in sets:
+                ctx.BindReshard(srcs, dsts)
+
+    def timed(with_laps):
+        """W warm-up steps, then exactly K steps: wall clock bracketed by synchronisation, HIP events on the
+        library's own stream for the device time inside it; then five more brackets of 50 launches and, with
+        `with_laps`, a timing mark between each two of at least 50 more launches."""
+        for i in range(args.warmup):
+            step(i)
+        ctx.Sync()
+        syncs_before = ctx.stats["host_blocking_syncs"]
+        t0 = time.perf_counter()
+        ctx.StartTimer()
+        for i in range(args.steps):
+            step(i)
+        syncs = ctx.stats["host_blocking_syncs"] - syncs_before  # waits the K reshards themselves caused
+        kernel_ms = ctx.StopTimer()  # blocks until the device gets there (a counted wait, asked for here)
+        ctx.Sync()
+        wall_s = time.perf_counter() - t0
+        brackets = []
+        for _ in range(5):
+            ctx.StartTimer()
+            for i in range(50):
+                step(i)
+            brackets.append(ctx.StopTimer() / 50)
+        brackets.sort()
+        laps = []
+        if with_laps:
+            n_laps = max(50, min(args.steps, 500))
+            ctx.Lap()
+            for i in range(n_laps):
+                step(i)
+                ctx.Lap()
+            laps = sorted(ctx.Laps())
+        return {"kernel_ms": kernel_ms / args.steps, "wall_s": wall_s, "syncs": syncs, "brackets": brackets, "laps": laps}
+
+    # the planner's own launch order first ...
+    bind_all()
+    untuned = timed(with_laps=not (args.tune and not args.unbatched))
+    run = untuned
     order_used = 0
+    # ... then, on request, the order mmr_reshard_tune keeps after timing a few on the first buffer set (a caller does
+    # this once, where it builds its schedule); measured again only if it kept another order than the default
     if args.tune and not args.unbatched:
         order_used = ctx.TuneReshard(sets[0][0], sets[0][1])
-    if not args.unbatched:
-        for srcs, dsts in sets:
-            ctx.BindReshard(srcs, dsts)
-    if args.tune and not args.unbatched:  # whatever order was kept, the bytes are the oracle's
-        step(0)
-        ctx.Sync()
-        check_parity(ctx, arrays, gs, sets[0][1], sample_only=alg_bytes > (2 << 30))
-
-    for i in range(args.warmup):
-        step(i)
-    ctx.Sync()
-    syncs_before = ctx.stats["host_blocking_syncs"]
-    # timed region: exactly K steps, wall clock bracketed by synchronisation;
-    # HIP events on the library's own stream give the device time inside it
-    t0 = time.perf_counter()
-    ctx.StartTimer()
-    for i in range(args.steps):
-        step(i)
-    syncs_in_region = ctx.stats["host_blocking_syncs"] - syncs_before  # waits the K reshards themselves caused
-    kernel_ms = ctx.StopTimer()  # blocks until the device gets there (a counted wait, asked for here)
-    ctx.Sync()
-    wall_s = time.perf_counter() - t0
-    # the same bracket five more times over 50 back-to-back launches each: the median of the five means
-    brackets = []
-    for _ in range(5):
-        ctx.StartTimer()
-        for i in range(50):
-            step(i)
-        brackets.append(ctx.StopTimer() / 50)
-    brackets.sort()
-    # per-launch distribution: a timing mark between each two of at least 50 back-to-back launches
-    n_laps = max(50, min(args.steps, 500))
-    ctx.Lap()
-    for i in range(n_laps):
-        step(i)
-        ctx.Lap()
-    laps = sorted(ctx.Laps())
+        if order_used != 0:
+            bind_all()
+            step(0)
+            ctx.Sync()
+            check_parity(ctx, arrays, gs, sets[0][1], sample_only=alg_bytes > (2 << 30))  # same bytes, whatever order
+        run = timed(with_laps=True)  # the kept order (the default's second measurement if nothing else was kept)
+    kernel_ms, wall_s, syncs_in_region = run["kernel_ms"] * args.steps, run["wall_s"], run["syncs"]
+    brackets, laps = run["brackets"], run["laps"]
 
     batched = len(arrays) > 1 and not args.unbatched
     plan = (ctx.plan_stats(sets[0][0][0], sets[0][1][0]) if single else
@@ -227,6 +243,9 @@ def measure(ctx, mm, workloads, args, config):
         "kernel": kernel, "n_arrays": len(arrays), "sets": len(sets), "order_used": order_used,
         "orders_timed": plan["orders_timed"] if plan else 0, "parity_arrays": checked,
         "host_blocking_syncs_in_timed_region": syncs_in_region,
+        # the same protocol with the planner's default launch order (what a caller gets who never calls mmr_reshard_tune)
+        "untuned_kernel_ms": untuned["kernel_ms"], "untuned_achieved": alg_bytes / (untuned["kernel_ms"] * 1e-3) / 1e9,
+        "untuned_bracket_median_ms": untuned["brackets"][2],
     }
     first_dsts = sets[0][1]
     for srcs, dsts in sets[1:]:
@@ -329,7 +348,9 @@ def summary(r):
             "median_GB/s": round(r["median_gbs"], 1), "algorithmic_bytes": r["alg_bytes"],
             "launches_per_step": r["launches"], "kernel": r["kernel"], "buffer_sets": r["sets"],
             "plan_build_ms_cold": round(r["plan_build_ms"], 3), "plan_table_bytes": r["plan_table_bytes"],
-            "order_used": r["order_used"], "orders_timed": r["orders_timed"], "parity_arrays_checked": r["parity_arrays"]}
+            "order_used": r["order_used"], "orders_timed": r["orders_timed"], "parity_arrays_checked": r["parity_arrays"],
+            "untuned_kernel_ms": round(r["untuned_kernel_ms"], 5), "untuned_GB/s": round(r["untuned_achieved"], 1),
+            "untuned_frac_hbm_peak": round(r["untuned_achieved"] / HBM_PEAK_GBS, 4)}
 
 
 def main():
@@ -430,6 +451,9 @@ def main():
             "bracket_median_ms": round(res["bracket_median_ms"], 5), "bracket_min_ms": round(res["bracket_min_ms"], 5),
             "bracket_max_ms": round(res["bracket_max_ms"], 5),
             "launches_per_step": res["launches"],
+            # the planner's default launch order, measured with the same protocol before mmr_reshard_tune ran
+            "untuned_kernel_ms": round(res["untuned_kernel_ms"], 5),
+            "untuned_frac": round(res["untuned_achieved"] / HBM_PEAK_GBS, 4), "order_used": res["order_used"],
             # the same launch priced at the bytes the HBM counters saw instead of the algorithmic ones
             "traffic_over_algorithmic": round(traffic / res["alg_bytes"], 4) if traffic else None,
             "counter_GB/s": round(traffic / (res["kernel_ms"] * 1e-3) / 1e9, 1) if traffic else None,
