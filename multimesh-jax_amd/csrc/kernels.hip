@@ -100,7 +100,18 @@ __device__ __forceinline__ gchar* slot_base(void* const* __restrict__ ptrs, uint
 }
 
 // Launch shape of the aligned kernel: 256 threads, 2 vectors each (8 KiB per workgroup), nontemporal both ways.
-constexpr int kCopy16Unroll = 2;
+// Measured against it on MI355X (bf16 [8,4096,8192] hidden 8-way -> sequence 4-way, 160.6 us): 512 threads x 1 vector
+// 222 us - every wave decodes its chunk on the scalar unit (some 200 scalar instructions), and with twice the waves
+// per byte the scalar unit, 53 % busy at 256 x 2, is the bound; 128 threads x 4 vectors 169 us.  A stand-alone copy of
+// the same access pattern whose chunk falls out of three shifts runs in 169 us at 256 x 2 and 160-162 us at 512 x 1.
+#ifndef MMR_COPY16_THREADS
+#define MMR_COPY16_THREADS 256
+#endif
+#ifndef MMR_COPY16_UNROLL
+#define MMR_COPY16_UNROLL 2
+#endif
+constexpr int kCopy16Threads = MMR_COPY16_THREADS;
+constexpr int kCopy16Unroll = MMR_COPY16_UNROLL;
 constexpr bool kCopy16NtLoads = true;
 
 // Translation prefetch.  A launch streams through its buffers once, so every 2 MiB page is new when the first
@@ -413,10 +424,10 @@ hipError_t launch_copy_groups(const CopyGroup* d_groups, uint32_t n_groups, cons
   GroupStarts s;
   for (uint32_t i = 0; i < kMaxDirectGroups; ++i) s.first[i] = starts && i < n_groups ? starts[i] : 0xffffffffu;
   if (starts && n_groups <= kMaxDirectGroups)
-    hipLaunchKernelGGL((mmr_copy16_kernel<256, kCopy16Unroll, true>), dim3(grid_size(n, group)), dim3(256), 0, stream,
+    hipLaunchKernelGGL((mmr_copy16_kernel<kCopy16Threads, kCopy16Unroll, true>), dim3(grid_size(n, group)), dim3(kCopy16Threads), 0, stream,
                        d_groups, n_groups, d_pieces, d_hints, static_cast<uint32_t>(n), group, s);
   else
-    hipLaunchKernelGGL((mmr_copy16_kernel<256, kCopy16Unroll, false>), dim3(grid_size(n, group)), dim3(256), 0, stream,
+    hipLaunchKernelGGL((mmr_copy16_kernel<kCopy16Threads, kCopy16Unroll, false>), dim3(grid_size(n, group)), dim3(kCopy16Threads), 0, stream,
                        d_groups, n_groups, d_pieces, d_hints, static_cast<uint32_t>(n), group, s);
   return hipGetLastError();
 }
@@ -427,7 +438,7 @@ hipError_t launch_copy_groups_inline(const InlineCopyTable& table, uint32_t xcd_
   if (hipError_t e = check_grid(n)) return e;
   if (table.n_groups > kInlineCopyGroups) return hipErrorInvalidValue;
   const uint32_t group = xcd_group_of(n, xcd_mode);
-  hipLaunchKernelGGL((mmr_copy16_inline_kernel<256, kCopy16Unroll>), dim3(grid_size(n, group)), dim3(256), 0, stream,
+  hipLaunchKernelGGL((mmr_copy16_inline_kernel<kCopy16Threads, kCopy16Unroll>), dim3(grid_size(n, group)), dim3(kCopy16Threads), 0, stream,
                      table, group);
   return hipGetLastError();
 }
