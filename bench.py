@@ -294,8 +294,16 @@ def record_traffic(args):
                         "dispatches": len(values), "scale": scale}
     alg = workloads.algorithmic_bytes(workloads.config(args.config))
     hbm = int((out["FETCH_SIZE"]["kib_mean"] * FETCH_SCALE + out["WRITE_SIZE"]["kib_mean"] * WRITE_SCALE) * 1024)
+    import subprocess
+    try:  # the commit whose sources the counters were measured on (the digest is what bench.py checks)
+        commit = subprocess.check_output(["git", "-C", ROOT, "rev-parse", "HEAD"], stderr=subprocess.DEVNULL).decode().strip()
+        if subprocess.call(["git", "-C", ROOT, "diff", "--quiet", "HEAD", "--", "multimesh-jax_amd/csrc", "include"]) != 0:
+            commit += " + uncommitted changes"
+    except Exception:
+        commit = None
     prof = {"config": args.config, "kernel": kernel, "counters": out, "hbm_bytes_per_launch": hbm,
             "algorithmic_bytes": alg, "ratio": round(hbm / alg, 4), "kernel_sources_digest": kernel_sources_digest(),
+            "measured_at_commit": commit,
             "source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, one counter per run, KiB per dispatch; "
                       "FETCH_SIZE x %.3f, WRITE_SIZE x %.3f" % (FETCH_SCALE, WRITE_SCALE)}
     path = os.path.join(ROOT, "profiles", "traffic_config%d.json" % args.config)
