@@ -355,10 +355,15 @@ void HipExecuteContext::OffloadDtoH(int64_t local_device_id, const std::vector<S
   int64_t seq = 0;
   (void)Arrive(kOffloadDtoH, local_device_id, &first, &seq);
   if (first) {
-    FlushLocked();
-    for (const StoreHandle& h : to_offload) {
-      require_live(h, "OffloadDtoH");
-      check(mmr_store_offload(ctx_, h.impl->array->store), "OffloadDtoH");
+    try {
+      FlushLocked();
+      for (const StoreHandle& h : to_offload) {
+        require_live(h, "OffloadDtoH");
+        check(mmr_store_offload(ctx_, h.impl->array->store), "OffloadDtoH");
+      }
+    } catch (...) {
+      Retract(kOffloadDtoH, local_device_id);  // the failed call consumed no position: the devices stay in step
+      throw;
     }
   }
   Leave(kOffloadDtoH);
@@ -372,10 +377,15 @@ void HipExecuteContext::OffloadHtoD(int64_t local_device_id, const std::vector<S
   int64_t seq = 0;
   (void)Arrive(kOffloadHtoD, local_device_id, &first, &seq);
   if (first) {
-    FlushLocked();
-    for (const StoreHandle& h : to_offload) {
-      require_live(h, "OffloadHtoD");
-      check(mmr_store_reload(ctx_, h.impl->array->store), "OffloadHtoD");
+    try {
+      FlushLocked();
+      for (const StoreHandle& h : to_offload) {
+        require_live(h, "OffloadHtoD");
+        check(mmr_store_reload(ctx_, h.impl->array->store), "OffloadHtoD");
+      }
+    } catch (...) {
+      Retract(kOffloadHtoD, local_device_id);  // the failed call consumed no position: the devices stay in step
+      throw;
     }
   }
   Leave(kOffloadHtoD);
