@@ -660,15 +660,16 @@ int get_plan(mmr_context* ctx, const std::vector<mmr_sharded_shape>& srcs, const
   *out = dp.get();
   ctx->plans.emplace(key, std::move(dp));
   ctx->plan_lru.push_front(std::move(key));
-  // Least recently used plans go when the cache is full.  Plans with bindings stay until mmr_context_clear_plans (a
-  // captured graph may hold their tables).
+  // Least recently used plans go when the cache is full; the device tables of one that goes return to the block pool,
+  // whose next user is ordered on the stream behind the launches that still read them.  Plans with bindings stay
+  // until mmr_context_clear_plans (a captured graph may hold their tables).
   if (ctx->plans.size() > kMaxPlans) {
     for (auto pos = std::prev(ctx->plan_lru.end()); pos != ctx->plan_lru.begin();) {
       auto victim = ctx->plans.find(*pos);
       auto prev = std::prev(pos);
       bool bound = false;
       for (const auto& b : ctx->bindings) bound |= b->plan == victim->second.get();
-      if (!bound && !victim->second->d_generic && !victim->second->d_transposes) {
+      if (!bound) {
         if (ctx->last_plan == victim->second.get()) forget_last_plan(ctx);
         ctx->plans.erase(victim);
         ctx->plan_lru.erase(pos);
@@ -1284,14 +1285,17 @@ void mmr_context_destroy(mmr_context* ctx) {
   if (!ctx) return;
   (void)hipSetDevice(ctx->device);
   if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
-  // every host function of the stream has run by now, so every callback is queued: the thread runs them and ends
+  // Every host function of the stream has run by now, so every callback is queued.  The thread ends once it has run
+  // them all, including those that a callback queued in turn (run_after counts them before it returns).
   if (ctx->callback_thread.joinable()) {
     {
-      std::lock_guard<std::mutex> lock(ctx->callback_mu);
+      std::unique_lock<std::mutex> lock(ctx->callback_mu);
+      ctx->callback_cv.wait(lock, [&] { return ctx->callbacks_done >= ctx->callbacks_queued; });
       ctx->callback_stop = true;
     }
     ctx->callback_cv.notify_all();
     ctx->callback_thread.join();
+    if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);  // work the last callbacks queued
   }
   for (auto& b : ctx->bindings) give_block(ctx, b->d_block, b->capacity);
   ctx->bindings.clear();
@@ -1494,20 +1498,28 @@ int mmr_clear_store_cache(mmr_context* ctx) {
   std::lock_guard<std::mutex> lock(ctx->mu);
   if (int rc = use_device(ctx)) return rc;
   if (int rc = refuse_capture(ctx, "mmr_clear_store_cache")) return rc;
-  for (auto& c : ctx->buffer_cache) {
-    for (auto& b : c.second) {
-      MMR_HIP(hipFree(b.base));
+  // a buffer leaves its list before it is freed, so a failure part-way leaves the lists true
+  bool freed = false;
+  for (auto& c : ctx->buffer_cache)
+    while (!c.second.empty()) {
+      const CachedBuffer b = c.second.back();
+      c.second.pop_back();
+      MMR_HIP(hipFree(b.base));  // waits for the device
       ctx->stats.bytes_allocated -= static_cast<int64_t>(b.bytes);
+      freed = true;
     }
-  }
   ctx->buffer_cache.clear();
   for (auto& c : ctx->free_pool)
-    for (char* b : c.second) {
+    while (!c.second.empty()) {
+      char* b = c.second.back();
+      c.second.pop_back();
+      ctx->free_pool_bytes -= c.first;
       MMR_HIP(hipFree(b));
       ctx->stats.bytes_allocated -= static_cast<int64_t>(c.first);
+      freed = true;
     }
   ctx->free_pool.clear();
-  ctx->free_pool_bytes = 0;
+  if (freed) ctx->stats.host_blocking_syncs += 1;
   bool any_host = false;
   for (auto& c : ctx->host_cache) any_host |= !c.second.empty();
   if (any_host)
@@ -1664,19 +1676,25 @@ int mmr_store_offload(mmr_context* ctx, mmr_store* store) {
   // a pinned buffer from the host cache of this descriptor, else a new one (allocated pinned, never registered
   // after the fact)
   std::vector<CachedBuffer>& pool = ctx->host_cache[store->shape_key];
+  char* host = nullptr;
   if (!pool.empty()) {
-    store->host = pool.back().base;
+    host = pool.back().base;
     pool.pop_back();
     ctx->stats.host_cache_hits += 1;
   } else {
     if (int rc = refuse_capture(ctx, "offloading a store that needs a new pinned buffer")) return rc;
-    MMR_HIP(hipHostMalloc(reinterpret_cast<void**>(&store->host), store->bytes, hipHostMallocDefault));
+    MMR_HIP(hipHostMalloc(reinterpret_cast<void**>(&host), store->bytes, hipHostMallocDefault));
     ctx->stats.host_bytes_allocated += static_cast<int64_t>(store->bytes);
     ctx->stats.host_bytes_high_watermark = std::max(ctx->stats.host_bytes_high_watermark, ctx->stats.host_bytes_allocated);
   }
   // ordered on the stream behind whatever produced the store (the `pipelined` stores of OffloadDtoH included); the
   // device buffer goes to the device cache at once: its next user is ordered on the same stream behind this copy
-  MMR_HIP(hipMemcpyAsync(store->host, store->base, store->bytes, hipMemcpyDeviceToHost, ctx->stream));
+  const hipError_t e = hipMemcpyAsync(host, store->base, store->bytes, hipMemcpyDeviceToHost, ctx->stream);
+  if (e != hipSuccess) {  // the store stays on the device; the pinned buffer is kept for the next offload
+    pool.push_back(CachedBuffer{host, store->bytes});
+    return fail(MMR_HIP_ERROR, "copy of store %lld to host memory failed: %s", (long long)store->id, hipGetErrorString(e));
+  }
+  store->host = host;
   ctx->buffer_cache[store->shape_key].push_back(CachedBuffer{store->base, store->bytes});
   store->base = nullptr;
   return MMR_OK;
@@ -1691,16 +1709,22 @@ int mmr_store_reload(mmr_context* ctx, mmr_store* store) {
   if (int rc = use_device(ctx)) return rc;
   hash_op(ctx, 7 /* OffloadHtoD */, {static_cast<uint64_t>(store->ordinal)});
   std::vector<CachedBuffer>& parked = ctx->buffer_cache[store->shape_key];
+  char* base = nullptr;
   if (!parked.empty()) {
-    store->base = parked.back().base;
+    base = parked.back().base;
     parked.pop_back();
     ctx->stats.cache_hits += 1;
   } else {
     if (int rc = refuse_capture(ctx, "reloading a store that needs new device memory")) return rc;
-    if (int rc = device_alloc(ctx, reinterpret_cast<void**>(&store->base), store->bytes)) return rc;
+    if (int rc = device_alloc(ctx, reinterpret_cast<void**>(&base), store->bytes)) return rc;
     account_alloc(ctx, static_cast<int64_t>(store->bytes));
   }
-  MMR_HIP(hipMemcpyAsync(store->base, store->host, store->bytes, hipMemcpyHostToDevice, ctx->stream));
+  const hipError_t e = hipMemcpyAsync(base, store->host, store->bytes, hipMemcpyHostToDevice, ctx->stream);
+  if (e != hipSuccess) {  // the store stays offloaded; the device buffer is kept for the next reload
+    parked.push_back(CachedBuffer{base, store->bytes});
+    return fail(MMR_HIP_ERROR, "copy of store %lld back to the device failed: %s", (long long)store->id, hipGetErrorString(e));
+  }
+  store->base = base;
   // the pinned buffer goes to the host cache at once: the next offload into it is ordered behind this copy
   ctx->host_cache[store->shape_key].push_back(CachedBuffer{store->host, store->bytes});
   store->host = nullptr;
@@ -2012,6 +2036,7 @@ int mmr_reshard_batch_plan_stats(mmr_context* ctx, mmr_store* const* srcs, mmr_s
   std::vector<mmr_sharded_shape> s, d;
   shapes_of(srcs, dsts, n, &s, &d);
   if (int rc = use_device(ctx)) return rc;
+  note_work(ctx);  // a plan built here uploads its tables
   DevicePlan* dp = nullptr;
   if (int rc = get_plan(ctx, s, d, &dp)) return rc;
   *out = dp->plan.stats;

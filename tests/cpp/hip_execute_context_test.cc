@@ -604,6 +604,28 @@ static int run() {
     EXPECT(h1 != 0 && h1 == h2 && h1 != h3);
   }
 
+  // A context that goes away with callbacks still waiting runs them all first - also the one a callback queued in
+  // its turn, behind a reshard it issued.
+  {
+    std::atomic<int> ran{0};
+    {
+      auto dc = HipExecuteContext::Create({0, 1});
+      ShardedShape a{SupportedType::F32, {{{64, 2, 0}, {32, 1, 1}}, DeviceList::Create(0, 2)}, {}};
+      ShardedShape b{SupportedType::F32, {{{64, 1, 0}, {32, 2, 1}}, DeviceList::Create(0, 2)}, {}};
+      std::vector<StoreHandle> x(2), y(2);
+      for (int d = 0; d < 2; ++d) x[d] = dc->CreateStore(d, d, a);
+      for (int d = 0; d < 2; ++d) y[d] = dc->CreateStore(d, d, b);
+      for (int d = 0; d < 2; ++d) dc->Reshard(d, d, x[d], y[d]);
+      HipExecuteContext* raw = dc.get();
+      dc->RunAfterAllTasks(0, [&ran, raw, x, y] {
+        ran.fetch_add(1);
+        for (int d = 0; d < 2; ++d) raw->Reshard(d, d, x[d], y[d]);
+        raw->RunAfterAllTasks(0, [&ran] { ran.fetch_add(10); });
+      });
+    }
+    EXPECT(ran.load() == 11);
+  }
+
   std::printf("OK\n");
   return 0;
 }

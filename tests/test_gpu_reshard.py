@@ -385,6 +385,44 @@ def test_plan_and_binding_caches(ctx):
         ctx.Free(st)
 
 
+def test_plan_cache_stays_bounded_when_plans_hold_device_tables():
+    """More distinct ragged descriptor pairs than the plan cache holds, each with chunk tables in device memory: the
+    least recently used plans go (their tables return to the block pool, where the later plans find theirs), and a
+    pair whose plan went is planned again with the same bytes."""
+    say("plan cache eviction with device tables")
+    with mm.ReshardContext(0) as ctx:
+        ctx.set_plan_options(0, 0, 0, B.MMR_PLAN_NO_SPAN)  # ragged boxes as generic chunks: a device table per plan
+
+        def case(rows):
+            return [{"name": "evict%d" % rows, "type": "U8", "shape": (rows, 37),
+                     "src": {"dims": [(rows, 1, 0), (37, 2, 1)], "dev_start": 0, "dev_count": 2},
+                     "dst": {"dims": [(rows, 1, 0), (37, 3, 1)], "dev_start": 4, "dev_count": 3},
+                     "seed": rows, "dist": "raw"}]
+
+        first = case(5)
+        g_first = [workloads.generate(a) for a in first]
+        _compare(first, g_first, gpu_reshard(ctx, first, g_first))
+        built0 = ctx.stats["plans_built"]
+        pool_hits = None
+        for rows in range(6, 6 + 300):
+            arrays = case(rows)
+            gs = [workloads.generate(a) for a in arrays]
+            srcs, dsts = make_stores(ctx, arrays, gs)
+            ctx.ReshardBatch(srcs, dsts)
+            if rows % 50 == 0:
+                _compare(arrays, gs, [read_all(ctx, d) for d in dsts])
+            for st in list(srcs) + list(dsts):
+                ctx.Free(st)
+            if rows == 6 + 269:  # the cache has been full for a while: tables now come from the pool
+                pool_hits = ctx.stats["block_pool_hits"]
+        st = ctx.stats
+        assert st["plans_built"] - built0 == 300
+        assert st["plans_cached"] <= 256
+        assert st["block_pool_hits"] - pool_hits >= 30  # one chunk table per plan at least
+        _compare(first, g_first, gpu_reshard(ctx, first, g_first))  # evicted long ago: planned again
+        assert ctx.stats["plans_built"] - built0 == 301
+
+
 def test_first_reshard_of_a_pair_does_not_wait_for_the_device():
     """A plain Reshard on descriptors never seen before plans, binds and launches without a single blocking
     synchronisation (the reference's Reshard is asynchronous), whichever launch classes the plan has; the plan it
