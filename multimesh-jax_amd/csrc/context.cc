@@ -861,8 +861,9 @@ int launch_block(mmr_context* ctx, const DevicePlan& dp, const char* block, cons
 }
 
 int64_t launches_of(const DevicePlan* dp) {
-  return (dp->plan.n_copy_chunks ? 1 : 0) + (dp->plan.n_span_chunks ? 1 : 0) + (dp->plan.generic.empty() ? 0 : 1) +
-         static_cast<int64_t>(dp->transpose_runs.size());
+  const uint32_t xm = dp->plan.options.xcd_mode == 0 ? 64 : dp->plan.options.xcd_mode;
+  return mmr::copy_group_launches(dp->plan.n_copy_chunks, xm) + (dp->plan.n_span_chunks ? 1 : 0) +
+         (dp->plan.generic.empty() ? 0 : 1) + static_cast<int64_t>(dp->transpose_runs.size());
 }
 
 // One launch per kernel class.  Tables in device memory, bound to these buffers, are the fast way (a workgroup's

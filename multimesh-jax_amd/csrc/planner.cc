@@ -223,7 +223,31 @@ class Builder {
     return out;
   }
 
+  // A run many chunks long (a box that is contiguous on both sides: a whole tile, a band of whole rows) becomes rows
+  // of one chunk each under a row dim of its own, so that one piece record serves the box; cut into column segments
+  // like a long row it would take one record per chunk (a 1 GiB tile: 131,072 records, 8 MB of tables).  What is
+  // left over behind the last whole row stays a box of its own.
+  void fold_long_runs() {
+    const int64_t row = chunk_bytes_;  // a multiple of 256
+    std::vector<CanonBox> tails;
+    for (CanonBox& b : tile_) {
+      if (b.outer.size() > 2 || b.w < 16 * row) continue;  // three row dims are blocked; more would multiply the groups
+      const int64_t n = b.w / row, rem = b.w % row;
+      if (rem) {
+        CanonBox tail = b;
+        tail.so = b.fill ? 0 : b.so + n * row;
+        tail.dof = b.dof + n * row;
+        tail.w = rem;
+        tails.push_back(std::move(tail));
+      }
+      b.outer.push_back(BoxDim{n, row, row});  // innermost: its rows abut on both sides
+      b.w = row;
+    }
+    for (CanonBox& t : tails) tile_.push_back(std::move(t));
+  }
+
   void lower_copy_groups() {
+    fold_long_runs();
     for (const std::vector<int>& mates : row_mates()) {
       const CanonBox& first = tile_[mates[0]];
       int64_t w_max = 0;

@@ -385,6 +385,35 @@ def test_plan_and_binding_caches(ctx):
         ctx.Free(st)
 
 
+def test_long_copy_tables_leave_in_pieces(ctx):
+    """A table of several hundred thousand copy chunks is launched as consecutive pieces of 131,072 chunks (long
+    launches lose bandwidth, a boundary restores it): the same bytes on the first launch on these buffers (device tables
+    are built) and on later ones (they are found)."""
+    say("long copy table in pieces")
+    ctx.set_plan_options(256, 0)  # 256-byte chunks: a long table over a small array
+    try:
+        arrays = workloads.config(2, 2)
+        gs = [workloads.generate(a) for a in arrays]
+        srcs, dsts = make_stores(ctx, arrays, gs)
+        chunks = ctx.plan_stats(srcs[0], dsts[0])["n_copy16_chunks"]
+        assert chunks >= 3 * 131072
+        pieces = -(-chunks // 131072)
+        for launch in range(2):
+            if launch:
+                junk = np.full(dsts[0].shard_bytes, 0xA5, dtype=np.uint8)
+                for dev in dsts[0].devices:
+                    ctx.AssembleShards(dsts[0].shape, dev, junk, existing_store=dsts[0])
+            before = ctx.stats
+            ctx.Reshard(srcs[0], dsts[0])
+            after = ctx.stats
+            assert after["kernel_launches"] - before["kernel_launches"] == pieces
+            _compare(arrays, gs, [read_all(ctx, dsts[0])])
+        for st in srcs + dsts:
+            ctx.Free(st)
+    finally:
+        ctx.set_plan_options(0, 0)
+
+
 def test_plan_cache_stays_bounded_when_plans_hold_device_tables():
     """More distinct ragged descriptor pairs than the plan cache holds, each with chunk tables in device memory: the
     least recently used plans go (their tables return to the block pool, where the later plans find theirs), and a

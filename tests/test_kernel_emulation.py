@@ -60,6 +60,31 @@ def test_chunk_sizes_wide_and_narrow_rows(chunk_bytes):
         _check(arrays, gs, chunk_bytes=chunk_bytes)
 
 
+@pytest.mark.parametrize("chunk_bytes", [256, 8192])
+def test_long_contiguous_runs_are_folded_into_rows(chunk_bytes):
+    """Tiles that are contiguous on both sides (the same dim sharded a different number of ways, whole rows regrouped)
+    are copied as rows of one chunk under one piece record each - the table does not grow with the tile - plus a
+    box for what is left behind the last whole row; a run under other row dims is folded the same way."""
+    tile = 20 * chunk_bytes + 48  # bytes per destination tile: 20 whole rows and a tail
+    cases = [
+        [{"name": "flat", "type": "U8", "shape": (3 * tile,),
+          "src": {"dims": [(3 * tile, 1, 0)], "dev_start": 0, "dev_count": 1},
+          "dst": {"dims": [(3 * tile, 3, 0)], "dev_start": 1, "dev_count": 3}, "seed": 1, "dist": "raw"}],
+        [{"name": "rows", "type": "F32", "shape": (96, tile // 16),
+          "src": {"dims": [(96, 2, 0), (tile // 16, 1, 1)], "dev_start": 0, "dev_count": 2},
+          "dst": {"dims": [(96, 3, 0), (tile // 16, 1, 1)], "dev_start": 2, "dev_count": 3}, "seed": 2, "dist": "raw"}],
+        # long rows that stay strided on the source side: a run of 40 chunks under a row dim
+        [{"name": "strided", "type": "U8", "shape": (6, 80 * chunk_bytes),
+          "src": {"dims": [(6, 1, 0), (80 * chunk_bytes, 2, 1)], "dev_start": 0, "dev_count": 2},
+          "dst": {"dims": [(6, 3, 0), (80 * chunk_bytes, 1, 1)], "dev_start": 2, "dev_count": 3}, "seed": 3, "dist": "raw"}],
+    ]
+    for arrays in cases:
+        gs = [workloads.generate(a) for a in arrays]
+        plan = _check(arrays, gs, chunk_bytes=chunk_bytes)
+        st = plan.stats
+        assert st["n_copy16_chunks"] >= 60 and st["n_pieces"] <= 12, (arrays[0]["name"], st)
+
+
 def test_traffic_of_the_headline_plan_is_exactly_algorithmic():
     from helpers import emulate_plan, lib_shape
     import multimesh_jax_amd as mm
