@@ -292,8 +292,19 @@ def record_traffic(args):
         kernel = name
         out[counter] = {"kib_mean": sum(values) / len(values), "kib_min": min(values), "kib_max": max(values),
                         "dispatches": len(values), "scale": scale}
-    alg = workloads.algorithmic_bytes(workloads.config(args.config))
-    hbm = int((out["FETCH_SIZE"]["kib_mean"] * FETCH_SCALE + out["WRITE_SIZE"]["kib_mean"] * WRITE_SCALE) * 1024)
+    arrays = workloads.config(args.config)
+    alg = workloads.algorithmic_bytes(arrays)
+    # a very long copy table leaves in several dispatches per launch (mmr_plan_stats.n_copy16_launches)
+    per_launch = 1
+    if "mmr_copy16" in kernel:
+        import multimesh_jax_amd as mm
+        def shape_of(type_, side):
+            return mm.sharded_shape(type_, side["dims"], side["dev_start"], side["dev_count"], side.get("minor_to_major"))
+        plan = mm.api.Plan([shape_of(a["type"], a["src"]) for a in arrays], [shape_of(a["type"], a["dst"]) for a in arrays])
+        per_launch = plan.stats["n_copy16_launches"]
+    for counter in out:
+        out[counter]["dispatches_per_launch"] = per_launch
+    hbm = int((out["FETCH_SIZE"]["kib_mean"] * FETCH_SCALE + out["WRITE_SIZE"]["kib_mean"] * WRITE_SCALE) * 1024 * per_launch)
     import subprocess
     try:  # the commit whose sources the counters were measured on (the digest is what bench.py checks)
         commit = subprocess.check_output(["git", "-C", ROOT, "rev-parse", "HEAD"], stderr=subprocess.DEVNULL).decode().strip()

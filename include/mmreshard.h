@@ -240,6 +240,7 @@ typedef struct {
   int64_t order_used;          /* table order in effect: 0 = the default mix, else a value of mmr_plan_options.order */
   int64_t interleave_kib;      /* order 4 only: KiB per tile and fraction */
   int64_t orders_timed;        /* how many launch orders mmr_reshard_tune timed for this plan (0 = never tuned) */
+  int64_t n_copy16_launches;   /* launches the copy-group table leaves in (very long tables go in pieces) */
 } mmr_plan_stats;
 
 int mmr_plan_create(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int32_t n_arrays,

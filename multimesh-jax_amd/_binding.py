@@ -87,7 +87,7 @@ class PlanStats(C.Structure):
         "n_arrays", "n_boxes", "n_copy16_chunks", "n_span_chunks", "n_groups", "n_pieces", "n_copy_generic_chunks",
         "n_transpose_chunks",
         "n_fill_chunks", "bytes_moved", "bytes_filled", "table_bytes", "n_slots", "order_used", "interleave_kib",
-        "orders_timed")]
+        "orders_timed", "n_copy16_launches")]
 
     def as_dict(self):
         return {n: getattr(self, n) for n, _ in self._fields_}

@@ -61,6 +61,41 @@ inline uint32_t grid_size(int64_t n, uint32_t group) {
   return static_cast<uint32_t>((n + span - 1) / span * span);
 }
 
+// Very long tables leave in pieces.  The eight XCDs do not work through their shares of a launch at the same rate
+// (0.5-1.5 % apart; start times of every workgroup of a 655,360-chunk launch, a probe build), so the workgroups in
+// flight spread over the table: 2,000 table positions at the start, 11,000 (90 MB) at the end of that launch, and
+// the rate falls with it: the hidden 8-way -> sequence 4-way split of bf16 [N, 4096, 8192] runs at 83 % of the 8
+// TB/s peak in one launch for N = 8 to 24 (65,536 to 196,608 chunks), at 81-82 % for N = 40 to 64 and at 80 % for N
+// = 80 (655,360 chunks, 10.7 GB).  A launch boundary brings the XCDs together again (the spread stays under 2,900
+// positions with pieces of 131,072) and costs 3-6 us.  Measured on
+// MI355X, pieces of 131,072 chunks (1 GiB read + 1 GiB written, ~0.33 ms) against one launch: N = 80 1.673 -> 1.641
+// ms, N = 64 1.313 -> 1.300 ms, N = 48 0.985 -> 0.977 ms, N = 40 0.825 -> 0.818 ms, a batch of 195 arrays (650 k
+// chunks) 1.706 -> 1.652 ms - within 1 % of what its arrays take one by one; 65,536 and 98,304 measure the same,
+// 196,608 and more gain less; N = 32 loses (0.675 -> 0.685 ms) and N <= 24 is unchanged or slower, so tables of
+// fewer than three pieces are launched whole.
+#ifndef MMR_COPY_PIECE_CHUNKS
+#define MMR_COPY_PIECE_CHUNKS 131072
+#endif
+#ifndef MMR_COPY_PIECES_MIN
+#define MMR_COPY_PIECES_MIN 3
+#endif
+
+// Chunks per launch of a copy-group table of n chunks (n itself: one launch).
+inline int64_t copy_piece_chunks(int64_t n, uint32_t xcd_mode) {
+  // a whole number of XCD rounds per piece, so that every piece but the last fills its grid exactly
+  const int64_t group = xcd_group_of(n, xcd_mode);
+  const int64_t unit = (group > 1 ? group : 1) * kXcds;
+  const int64_t piece = (static_cast<int64_t>(MMR_COPY_PIECE_CHUNKS) + unit - 1) / unit * unit;
+  if (xcd_mode == 2 || n < piece * MMR_COPY_PIECES_MIN) return n > 1 ? n : 1;
+  return piece;
+}
+
+inline int64_t copy_group_launches(int64_t n, uint32_t xcd_mode) {
+  if (n <= 0) return 0;
+  const int64_t piece = copy_piece_chunks(n, xcd_mode);
+  return (n + piece - 1) / piece;
+}
+
 // ---------------------------------------------------------------------------
 // Aligned copy: every offset, stride and row width is a multiple of 16 bytes.
 // Rows of wv = w/16 vectors.  The (row, column) pairs of the chunk are numbered

@@ -22,10 +22,8 @@ hipError_t launch_flat_copy(const void* src, void* dst, size_t bytes, hipStream_
 hipError_t launch_copy_groups(const CopyGroup* d_groups, uint32_t n_groups, const CopyPiece* d_pieces,
                               const uint32_t* d_hints, const uint32_t* starts, int64_t n, uint32_t xcd_mode,
                               hipStream_t stream);
-// Tables of very many chunks leave as several launches over consecutive pieces of the table (kernels.hip says why):
-// the chunks per piece, and the launches launch_copy_groups / launch_copy_groups_inline make for n chunks.
-int64_t copy_piece_chunks(int64_t n, uint32_t xcd_mode);
-int64_t copy_group_launches(int64_t n, uint32_t xcd_mode);
+// Tables of very many chunks leave as several launches over consecutive pieces of the table (copy_piece_chunks,
+// chunk_ops.h).
 // The same for a table small enough to travel in the kernel's argument block.
 hipError_t launch_copy_groups_inline(const InlineCopyTable& table, uint32_t xcd_mode, hipStream_t stream);
 // Span groups (ragged rows into dense destination tiles), staged through LDS.

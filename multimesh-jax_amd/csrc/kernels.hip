@@ -131,22 +131,6 @@ constexpr bool kCopy16NtLoads = true;
 constexpr uint32_t kPrefetchAhead = MMR_PREFETCH_AHEAD;  // chunks; 0 = off
 constexpr uint32_t kPrefetchEvery = MMR_PREFETCH_EVERY;  // a prime, so that every piece of a row block gets its turn
 
-// Very long tables leave in pieces.  The longer a launch runs, the further its waves spread over the table, and its
-// rate falls with it: the hidden 8-way -> sequence 4-way split of bf16 [N, 4096, 8192] runs at 83 % of the 8 TB/s
-// peak in one launch for N = 8 to 24 (65,536 to 196,608 chunks), at 81-82 % for N = 40 to 64 and at 80 % for N = 80
-// (655,360 chunks, 10.7 GB).  A launch boundary brings the waves together again and costs 3-6 us.  Measured on
-// MI355X, pieces of 131,072 chunks (1 GiB read + 1 GiB written, ~0.33 ms) against one launch: N = 80 1.673 -> 1.641
-// ms, N = 64 1.313 -> 1.300 ms, N = 48 0.985 -> 0.977 ms, N = 40 0.825 -> 0.818 ms, a batch of 195 arrays (650 k
-// chunks) 1.706 -> 1.652 ms - within 1 % of what its arrays take one by one; 65,536 and 98,304 measure the same,
-// 196,608 and more gain less; N = 32 loses (0.675 -> 0.685 ms) and N <= 24 is unchanged or slower, so tables of
-// fewer than three pieces are launched whole.
-#ifndef MMR_COPY_PIECE_CHUNKS
-#define MMR_COPY_PIECE_CHUNKS 131072
-#endif
-#ifndef MMR_COPY_PIECES_MIN
-#define MMR_COPY_PIECES_MIN 3
-#endif
-
 // Copy groups: the workgroup works its chunk out from the group table (bound: absolute addresses).  `groups` and
 // `pieces` are wave-uniform reads (scalar loads); the records are taken by value so that their loads leave together.
 template <int THREADS, int UNROLL, class FindGroup>
@@ -432,20 +416,6 @@ hipError_t launch_flat_copy(const void* src, void* dst, size_t bytes, hipStream_
   return hipGetLastError();
 }
 
-int64_t copy_piece_chunks(int64_t n, uint32_t xcd_mode) {
-  // a whole number of XCD rounds per piece, so that every piece but the last fills its grid exactly
-  const int64_t unit = static_cast<int64_t>(std::max<uint32_t>(xcd_group_of(n, xcd_mode), 1)) * kXcds;
-  const int64_t piece = (static_cast<int64_t>(MMR_COPY_PIECE_CHUNKS) + unit - 1) / unit * unit;
-  if (xcd_mode == 2 || n < piece * MMR_COPY_PIECES_MIN) return std::max<int64_t>(n, 1);
-  return piece;
-}
-
-int64_t copy_group_launches(int64_t n, uint32_t xcd_mode) {
-  if (n <= 0) return 0;
-  const int64_t piece = copy_piece_chunks(n, xcd_mode);
-  return (n + piece - 1) / piece;
-}
-
 hipError_t launch_copy_groups(const CopyGroup* d_groups, uint32_t n_groups, const CopyPiece* d_pieces,
                               const uint32_t* d_hints, const uint32_t* starts, int64_t n, uint32_t xcd_mode,
                               hipStream_t stream) {
@@ -454,7 +424,7 @@ hipError_t launch_copy_groups(const CopyGroup* d_groups, uint32_t n_groups, cons
   const uint32_t group = xcd_group_of(n, xcd_mode);
   GroupStarts s;
   for (uint32_t i = 0; i < kMaxDirectGroups; ++i) s.first[i] = starts && i < n_groups ? starts[i] : 0xffffffffu;
-  const int64_t piece = copy_piece_chunks(n, xcd_mode);
+  const int64_t piece = copy_piece_chunks(n, xcd_mode);  // long tables leave in pieces (chunk_ops.h says why)
   for (int64_t first = 0; first < n; first += piece) {
     const uint32_t grid = grid_size(std::min(piece, n - first), group);
     if (starts && n_groups <= kMaxDirectGroups)

@@ -943,6 +943,7 @@ int build_plan(const mmr_sharded_shape* srcs, const mmr_sharded_shape* dsts, int
   plan->stats.interleave_kib = options.order == 4 ? (fraction_kib ? fraction_kib : 64) : 0;
   plan->stats.n_arrays = n;
   plan->stats.n_copy16_chunks = plan->n_copy_chunks;
+  plan->stats.n_copy16_launches = copy_group_launches(plan->n_copy_chunks, options.xcd_mode == 0 ? 64 : options.xcd_mode);
   plan->stats.n_span_chunks = plan->n_span_chunks;
   plan->stats.n_copy_generic_chunks = static_cast<int64_t>(plan->generic.size());
   plan->stats.n_transpose_chunks = static_cast<int64_t>(plan->transposes.size());
