@@ -461,7 +461,10 @@ int mmr_window_open(mmr_context* ctx);
 int mmr_window_close(mmr_context* ctx);
 int mmr_context_set_max_open_windows(mmr_context* ctx, int32_t n);
 
-/* Unnamed HIP-event stopwatch on the context's stream for benchmarks: one interval at a time. */
+/* Unnamed HIP-event stopwatch on the context's stream for benchmarks: one interval at a time.  The events behind
+ * every timer, mark and window marker of this library are made without the system-scope fence
+ * (hipEventDisableSystemFence): they tell time and completion and cost the device no cache write-back in the middle
+ * of a schedule; to read what the device wrote, wait with mmr_sync or read through mmr_store_read_shard. */
 int mmr_timer_start(mmr_context* ctx);
 int mmr_timer_stop_wait(mmr_context* ctx, float* milliseconds); /* blocks until the device reaches this point */
 /* Per-launch timing of back-to-back work: mmr_timer_lap records a mark on the stream (between two launches, say);

@@ -308,6 +308,10 @@ namespace {
 constexpr size_t kMaxPlans = 256;  // cached plans per context (least recently used go first)
 constexpr size_t kFreePoolLimit = static_cast<size_t>(16) << 30;  // bytes the allocator keeps before it really frees
 
+#ifndef MMR_TIMING_EVENT_FLAGS
+#define MMR_TIMING_EVENT_FLAGS (hipEventDefault | hipEventDisableSystemFence)
+#endif
+
 #define MMR_HIP(expr)                                                                             \
   do {                                                                                            \
     hipError_t e_ = (expr);                                                                       \
@@ -377,6 +381,10 @@ int blocking_wait(mmr_context* ctx, hipEvent_t e) {
   return MMR_OK;
 }
 
+// Events that only mark a point in time (timer marks, window markers, laps): nothing the host reads hangs on them, so
+// they need no system-scope fence - which would write back and invalidate the caches in the middle of a schedule.
+constexpr unsigned kTimingEventFlags = MMR_TIMING_EVENT_FLAGS;
+
 int take_event(mmr_context* ctx, bool timing, hipEvent_t* out) {
   std::vector<hipEvent_t>& pool = timing ? ctx->free_timing_events : ctx->free_plain_events;
   if (!pool.empty()) {
@@ -384,7 +392,7 @@ int take_event(mmr_context* ctx, bool timing, hipEvent_t* out) {
     pool.pop_back();
     return MMR_OK;
   }
-  MMR_HIP(hipEventCreateWithFlags(out, timing ? hipEventDefault : hipEventDisableTiming));
+  MMR_HIP(hipEventCreateWithFlags(out, timing ? kTimingEventFlags : hipEventDisableTiming));
   return MMR_OK;
 }
 
@@ -1268,8 +1276,8 @@ int mmr_context_create(int32_t hip_device, void* hip_stream, mmr_context** out) 
     MMR_HIP(hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking));  // default priority
     ctx->owns_stream = true;
   }
-  MMR_HIP(hipEventCreate(&ctx->t0));
-  MMR_HIP(hipEventCreate(&ctx->t1));
+  MMR_HIP(hipEventCreateWithFlags(&ctx->t0, kTimingEventFlags));
+  MMR_HIP(hipEventCreateWithFlags(&ctx->t1, kTimingEventFlags));
   MMR_HIP(hipHostMalloc(reinterpret_cast<void**>(&ctx->staging), kStagingBytes, hipHostMallocDefault));
   // set-up of the entry point that may not allocate: everything it needs exists from here on
   MMR_HIP(mmr::static_scratch_address(hip_device, reinterpret_cast<void**>(&ctx->static_scratch)));
@@ -1880,7 +1888,7 @@ int mmr_timer_lap(mmr_context* ctx) {
   std::lock_guard<std::mutex> lock(ctx->mu);
   if (ctx->laps_used == ctx->laps.size()) {
     hipEvent_t e = nullptr;
-    MMR_HIP(hipEventCreate(&e));
+    MMR_HIP(hipEventCreateWithFlags(&e, kTimingEventFlags));
     ctx->laps.push_back(e);
   }
   MMR_HIP(hipEventRecord(ctx->laps[ctx->laps_used], ctx->stream));
