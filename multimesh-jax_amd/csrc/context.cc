@@ -56,7 +56,11 @@ struct DevicePlan {
   size_t generic_capacity = 0, transposes_capacity = 0;
   bool inline_copy = false, inline_span = false;  // the group table fits the kernel's argument block
   uint64_t serial = 0;
-  uint64_t recent[8] = {};  // hashes of the buffer sets of the last launches that went without device tables
+  // Hashes of the buffer sets of the last launches that went without device tables.  As many as bindings are kept: a
+  // schedule whose fresh output stores come round from the allocator's pool in a longer cycle than this list holds
+  // would never see a set "again" and never get device tables (3 parameter sets x 4 output buffers in rotation
+  // make 12 combinations).
+  uint64_t recent[kMaxBindings] = {};
   uint32_t recent_at = 0;
 
   DevicePlan() = default;
@@ -894,7 +898,7 @@ int launch_plan(mmr_context* ctx, DevicePlan* dp, const std::vector<void*>& ptrs
     bool want = dp->needs_binding() || tables == 1;
     if (!want && !capturing(ctx)) {  // seen these buffers before?
       for (uint64_t r : dp->recent) want |= r == key;
-      if (!want) dp->recent[dp->recent_at++ % 8] = key;
+      if (!want) dp->recent[dp->recent_at++ % kMaxBindings] = key;
     }
     if (want)
       if (int rc = get_binding(ctx, dp, ptrs, /*pin=*/false, /*count_hit=*/false, &binding)) return rc;

@@ -604,6 +604,37 @@ static int run() {
     EXPECT(h1 != 0 && h1 == h2 && h1 != h3);
   }
 
+  // Output stores that come round in a longer cycle (the caller holds the results of the last three executions, the
+  // parameters alternate between three sets: 12 combinations of buffers): every combination gets its device tables
+  // the second time it is seen, after which no launch carries its tables in the kernel's argument block any more.
+  {
+    auto rc = HipExecuteContext::Create(local);
+    ReshardSchedule rotating("rotating");
+    const Store p = rotating.AddStore(Store::Type::PARAM, "p", src);
+    const Store r = rotating.AddStore(Store::Type::ROOT, "r", dst);
+    rotating.AddReshardTask(p, r);
+    std::vector<std::vector<std::vector<StoreHandle>>> sets(
+        3, std::vector<std::vector<StoreHandle>>(kLocal, std::vector<StoreHandle>(1)));
+    for (auto& set : sets)
+      for (int d = 0; d < kLocal; ++d) set[d][0] = rc->CreateStore(d, d, src);
+    std::vector<std::vector<std::vector<StoreHandle>>> keep(3);
+    int turn = 0;
+    auto execute = [&] {
+      auto roots = rotating.Execute(*rc, sets[turn % 3]);
+      keep[turn % 3] = std::move(roots);
+      ++turn;
+    };
+    for (int i = 0; i < 36; ++i) execute();
+    const mmr_context_stats r0 = rc->Stats();
+    for (int i = 0; i < 24; ++i) execute();
+    const mmr_context_stats r1 = rc->Stats();
+    EXPECT(r1.reshard_calls - r0.reshard_calls == 24);
+    EXPECT(r1.inline_launches == r0.inline_launches);
+    EXPECT(r1.bindings_built == r0.bindings_built);
+    EXPECT(r1.binding_cache_hits - r0.binding_cache_hits == 24);
+    EXPECT(r1.device_allocations == r0.device_allocations);
+  }
+
   // A context that goes away with callbacks still waiting runs them all first - also the one a callback queued in
   // its turn, behind a reshard it issued.
   {
