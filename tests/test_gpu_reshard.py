@@ -589,12 +589,14 @@ def test_event_ordering_entry_points(ctx):
     assert hip.hipEventDestroy(ev) == 0
 
 
-def test_reshard_replays_from_a_hip_graph():
+@pytest.mark.parametrize("long_table", [False, True])
+def test_reshard_replays_from_a_hip_graph(long_table):
     """Once its plan and pointer table are bound, a reshard is kernel launches only.
     Captured into a HIP graph, it is replayed three times with different data in the
     stores, eager work and synchronisations of the same context in between; every
     replay must match the oracle.  An unbound reshard during capture is refused
-    without breaking the capture."""
+    without breaking the capture.  `long_table`: a copy table long enough to leave
+    in four launches, which the graph holds as four kernel nodes."""
     import ctypes as C
     hip = C.CDLL("libamdhip64.so.7")  # the runtime the library already loaded
     for fn in (hip.hipStreamBeginCapture, hip.hipStreamEndCapture, hip.hipGraphInstantiate, hip.hipGraphLaunch,
@@ -609,10 +611,16 @@ def test_reshard_replays_from_a_hip_graph():
 
     ctx = mm.ReshardContext(0)  # a context of its own: a broken capture must not leak into other tests
     try:
-        # mixed plan: aligned chunks (configuration 2 scaled), ragged rows (configuration 5 scaled), transposed layout
-        arrays = workloads.config(2, 8) + workloads.config(5, 16) + workloads.config(13, 16)
+        if long_table:
+            ctx.set_plan_options(256, 0)  # 256-byte chunks: 524,288 of them for a 128 MiB array
+            arrays = workloads.config(2, 2)
+        else:
+            # mixed plan: aligned chunks (configuration 2 scaled), ragged rows (configuration 5 scaled), transposed layout
+            arrays = workloads.config(2, 8) + workloads.config(5, 16) + workloads.config(13, 16)
         gs = [workloads.generate(a) for a in arrays]
         srcs, dsts = make_stores(ctx, arrays, gs)
+        if long_table:
+            assert ctx.batch_plan_stats(srcs, dsts)["n_copy16_launches"] == 4
         other = workloads.config(1, 16)
         other_g = [workloads.generate(a) for a in other]
         other_srcs, other_dsts = make_stores(ctx, other, other_g)
