@@ -533,10 +533,11 @@ MMR_HD void span_table_gather(const SpanGroup& g, const SpanMember& m, const Spa
   constexpr int ITEMS = DEPTH + (kSpanAlignedLoads ? 2 : 1);
   // one pass unless the span is a full one in a buffer that is not 16-byte aligned (one vector more than LANES * DEPTH)
   for (uint32_t base = 0; base < n_a; base += LANES * DEPTH) {
-    V16 v[ITEMS];
-    uint32_t at[ITEMS];
-    bool live[ITEMS], zero[ITEMS], keep[ITEMS];
-    typename M::cptr from[ITEMS];
+    constexpr int SLOTS = DEPTH + 2;  // ITEMS of them are used
+    V16 v[SLOTS];
+    uint32_t at[SLOTS];
+    bool live[SLOTS], zero[SLOTS], keep[SLOTS];
+    typename M::cptr from[SLOTS];
 #pragma unroll
     for (int u = 0; u < DEPTH; ++u) {
       const uint32_t i = base + lane + u * LANES;
