@@ -50,6 +50,23 @@ def test_config4_full_size_plan_is_one_aligned_launch():
     assert s["n_transpose_chunks"] == 0 and s["n_copy_generic_chunks"] == 0 and s["n_fill_chunks"] == 0
     assert 2 * s["bytes_moved"] == 10_713_055_232 == workloads.algorithmic_bytes(arrays)
     assert s["n_slots"] == 195 * 12
+    # the table is long enough to leave in pieces of 131,072 chunks
+    assert s["n_copy16_chunks"] == 654_984 and s["n_copy16_launches"] == 5
+
+
+def test_only_tables_of_three_pieces_and_more_leave_in_pieces():
+    """Launch pieces of 131,072 chunks (measured: shorter tables lose by being cut); a contiguous tile costs two piece
+    records however long it is."""
+    for chunks, launches in ((65_536, 1), (262_144, 1), (393_214, 1), (393_216, 3), (400_000, 4), (655_360, 5)):
+        n = chunks * 8192
+        plan = mm.Plan(mm.sharded_shape("U8", [(n, 1, 0)], 0, 1), mm.sharded_shape("U8", [(n, 2, 0)], 1, 2))
+        s = plan.stats
+        assert s["n_copy16_chunks"] == chunks and s["n_copy16_launches"] == launches, (chunks, s)
+        assert s["n_pieces"] <= 4 and s["table_bytes"] < 64 * 1024, s
+    # each XCD a contiguous eighth of the table: one launch whatever the length
+    plan = mm.Plan(mm.sharded_shape("U8", [(655_360 * 8192, 1, 0)], 0, 1),
+                   mm.sharded_shape("U8", [(655_360 * 8192, 2, 0)], 1, 2), xcd_mode=2)
+    assert plan.stats["n_copy16_launches"] == 1
 
 
 def test_config2_full_size_plan_shape():
